@@ -62,6 +62,7 @@ class RequestEntry:
     reserved: int = 0  # tokens beyond num_tokens that have pages for the running step
     tables: list[list[int]] = dataclasses.field(default_factory=list)  # per group: page id or -1 per page index
     versions: list[int] = dataclasses.field(default_factory=list)  # per group: counts the changes of its table
+    steps: int = 0  # steps of this request that were committed (its state's phase: see CacheManager.run_state)
     serial: int = 0  # which life of which request this is: no two calls of add_request give the same
     freed_upto: list[int] = dataclasses.field(default_factory=list)  # per group: pages below this index (and beyond
     # the rule's kept prefix) have been given back
@@ -80,6 +81,7 @@ class CacheView:
     attn_meta: Optional[object] = None
     group: Optional[int] = None
     pages: Optional[dict] = None  # further per-token tensors of this run, by name: [pages, page_size, *shape]
+    run_state: Optional[dict] = None  # the arrangement's per-request state of this run, by name: [slots, 2, *shape]
 
 
 def group_key(need: CacheNeed):
@@ -179,6 +181,7 @@ class CacheManager:
         dtype: torch.dtype,
         device: torch.device | str,
         poison: bool = False,
+        run_states: Optional[dict] = None,
     ) -> None:
         if page_size < 1:
             raise ValueError("page_size must be positive")
@@ -209,6 +212,15 @@ class CacheManager:
                 self.state[cid] = torch.zeros(
                     (max_requests, *need.state_shape), dtype=need.state_dtype or torch.float32, device=self.device
                 )
+        # State that an arrangement keeps per run of the order (``run_states``: place in the order -> {name: (shape,
+        # dtype)}), in two halves: a step reads the half that the request's last committed step wrote and writes
+        # the other (``state_phase``), so a step that is run again before its commit - a recorded step is run
+        # once launch by launch first - reads what the first run read, and no row of a step reads what another
+        # row of the same step writes.
+        self.run_state: dict[int, dict[str, torch.Tensor]] = {}
+        for k, named in (run_states or {}).items():
+            self.run_state[k] = {name: torch.zeros((max_requests, 2, *shape), dtype=dt or torch.float32,
+                                                   device=self.device) for name, (shape, dt) in named.items()}
         fill = float("nan") if poison else 0.0
         for g in self.groups:
             for cid in g.cache_ids:
@@ -228,6 +240,9 @@ class CacheManager:
         slot = self.slots.alloc()
         for t in self.state.values():
             t[slot].zero_()
+        for named in self.run_state.values():
+            for t in named.values():
+                t[slot].zero_()
         self._lives += 1
         e = RequestEntry(slot=slot, tables=[[] for _ in self.groups], versions=[0 for _ in self.groups],
                          serial=self._lives, freed_upto=[0 for _ in self.groups])
@@ -289,6 +304,7 @@ class CacheManager:
         e = self.requests[rid]
         e.num_tokens += e.reserved
         e.reserved = 0
+        e.steps += 1
         for g in self.groups:
             keep_from = first_needed_position(g.retention, e.num_tokens)
             table = e.tables[g.index]
@@ -342,6 +358,10 @@ class CacheManager:
 
     def slot(self, rid) -> int:
         return self.requests[rid].slot
+
+    def state_phase(self, rid) -> int:
+        """Which half of its two-halved state the request's next step reads (it writes the other)."""
+        return self.requests[rid].steps & 1
 
     def table(self, rid, group: int) -> list[int]:
         return self.requests[rid].tables[group]

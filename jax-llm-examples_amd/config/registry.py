@@ -66,9 +66,11 @@ def architecture_name(top: Mapping[str, Any]) -> str:
     archs = top.get("architectures")
     if archs:
         return str(archs[0])
+    if top.get("architecture"):  # (one name, not a list)
+        return str(top["architecture"])
     if top.get("model_type"):  # (a folder written without the entry)
         return str(top["model_type"])
-    raise UnknownArchitectureError("config.json has neither an 'architectures' entry nor a 'model_type'")
+    raise UnknownArchitectureError("config.json has neither an 'architectures' (or 'architecture') entry nor a 'model_type'")
 
 
 def read_config_json(model_dir: str | os.PathLike) -> dict:
@@ -87,3 +89,4 @@ def load_config(model_dir: str | os.PathLike):
 def _ensure_builtin() -> None:
     # importing the module registers the built-in architecture
     from ..parts import llama4 as _llama4  # noqa: F401
+    from ..parts import rovidra as _rovidra  # noqa: F401

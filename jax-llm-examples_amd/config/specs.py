@@ -43,10 +43,12 @@ class LayerSpec:
     """One decoder layer: which parts it is made of and how they are arranged."""
 
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None  # None: the layer has no feed-forward (for arrangements that allow it)
     mixer_norm: PartSpec
     feed_forward_norm: PartSpec
     arrangement: str = "pre_norm"
+    # what an arrangement needs beyond the four parts (further norms, gates, a token shift): its own keys
+    options: Mapping[str, Any] = dataclasses.field(default_factory=dict)
 
 
 @dataclasses.dataclass(frozen=True)

@@ -58,6 +58,7 @@ class StepContext:
     cu_seqlens: torch.Tensor  # int32 [R + 1]
     context_lens: torch.Tensor  # int32 [R]: tokens of the request after this step
     state_slots: torch.Tensor  # int32 [R]
+    state_phase: torch.Tensor  # int32 [R]: the half of a two-halved per-request state that this step reads
     logits_indices: torch.Tensor  # int32 [M]
     groups: list[GroupContext]
     # host copies
@@ -84,7 +85,7 @@ class StepLayout:
         N, R = num_tokens, num_segments
         self.num_tokens, self.num_segments, self.num_wanted, self.widths = N, R, num_wanted, list(widths)
         fields = [("token_ids", N), ("positions", N), ("token_segment", N), ("cu_seqlens", R + 1),
-                  ("context_lens", R), ("state_slots", R), ("logits_indices", num_wanted)]
+                  ("context_lens", R), ("state_slots", R), ("state_phase", R), ("logits_indices", num_wanted)]
         for g, w in enumerate(self.widths):
             fields += [(f"block_table{g}", R * w), (f"slot_mapping{g}", N)]
         self.bounds, o = {}, 0
@@ -114,6 +115,7 @@ def fill_step(layout: StepLayout, flat: np.ndarray, cache, entries: Sequence[Ste
     v = lambda name: layout.view(flat, name)
     tok, pos, seg, cu = v("token_ids"), v("positions"), v("token_segment"), v("cu_seqlens")
     ctx_lens, slots, want = v("context_lens"), v("state_slots"), v("logits_indices")
+    phase = v("state_phase")
     tables = [v(f"block_table{g.index}") for g in cache.groups]
     maps = [v(f"slot_mapping{g.index}") for g in cache.groups]
     seg_lens, seg_starts = [], []
@@ -143,7 +145,7 @@ def fill_step(layout: StepLayout, flat: np.ndarray, cache, entries: Sequence[Ste
                 want[w] = o + x
             w += 1
         cu[i + 1] = o + n
-        ctx_lens[i], slots[i] = start + n, cache.slot(e.rid)
+        ctx_lens[i], slots[i], phase[i] = start + n, cache.slot(e.rid), cache.state_phase(e.rid)
         stamp = cache.table_stamp(e.rid) if stamps is not None else None
         fresh = stamps is None or stamps[i] != stamp
         for g, width, bt, sm in zip(cache.groups, layout.widths, tables, maps):
@@ -190,6 +192,7 @@ def context_over(layout: StepLayout, flat: torch.Tensor, cache, ops, dtype, devi
         ops=ops, dtype=dtype, device=torch.device(device), num_tokens=layout.num_tokens, num_segments=R,
         token_ids=d("token_ids"), positions=d("positions"), token_segment=d("token_segment"),
         cu_seqlens=d("cu_seqlens"), context_lens=d("context_lens"), state_slots=d("state_slots"),
+        state_phase=d("state_phase"),
         logits_indices=d("logits_indices"), groups=groups, seg_lens=seg_lens, seg_starts=seg_starts,
         max_seg_len=max(seg_lens), max_context_len=max_context_len, page_size=cache.page_size, tap=tap)
 

@@ -70,7 +70,7 @@ class Engine:
                                cache_tokens=cache_tokens, memory_bytes=memory)
         self.cache = CacheManager(needs, page_size=page_size, num_pages=num_pages,
                                   max_requests=decode_batch_size, dtype=model.dtype, device=model.device,
-                                  poison=poison)
+                                  poison=poison, run_states=model.run_state_needs())
         self.runner = ModelRunner(model, self.cache, self.ops, decode_graphs=decode_graphs)
         self.scheduler = Scheduler(SchedulerConfig(max_num_batched_tokens, decode_batch_size, keep_free_pages,
                                                    max_seq_len), self.cache)

@@ -39,7 +39,8 @@ def make_runner(model_dir: str, dtype, max_tokens: int, device: str = "cuda:0", 
     rounded = -(-max_tokens // 64) * 64
     num_pages = -(-rounded // page_size) + max_requests
     cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages,
-                         max_requests=max_requests, dtype=dtype, device=device, poison=poison)
+                         max_requests=max_requests, dtype=dtype, device=device, poison=poison,
+                         run_states=model.run_state_needs())
     return ModelRunner(model, cache, ops, decode_graphs=decode_graphs)
 
 

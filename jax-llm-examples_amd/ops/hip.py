@@ -57,6 +57,12 @@ _SIGNATURES = {
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _vp, _vp,
                         _vp],
+    "jle_add_norm_shift": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                           _vp, _i, _i, _i, _i, _vp],
+    "jle_polynorm": [_vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+    "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "jle_latent_attention": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i,
+                             _vp, _vp, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -195,7 +201,138 @@ class HipOps:
         self._call("jle_embed", _p(token_ids), _p(table), self._is_bf16(table), _p(out), n, d)
         return out
 
+    SHIFT_ROWS_PER_BLOCK = 8  # a block of the norm-and-shift kernel takes so many rows in a step of many tokens
+    # (it forms the row before its first anew)
+
+    def add_norm_shift(self, x, delta, weight, eps: float, out_dtype, shift, ctx, do_norm: bool = True):
+        """``x' = x + delta`` into a new tensor (``delta``: ``None``, a tensor, or a gated branch
+        ``rmsnorm((y + b) * sigmoid(g + c)) * w_b`` that the kernel forms on the fly), ``h = rmsnorm(x') * weight``
+        and, with ``shift = (w, state)``, ``hs = h + (h_prev - h) * w`` with the float32 ``h`` of the token before
+        (from the request's two-halved state across steps).  Returns ``(x', h, hs or None)``."""
+        n, d = x.shape
+        self._chk(x, torch.float32, (n, d), "residual")
+        delta = self.materialize(delta) if isinstance(delta, ExpertSum) else delta
+        kind, y, yb, g, gb, pw, peps = 0, None, None, None, None, None, 0.0
+        if hasattr(delta, "gate"):
+            kind, y, yb, g, gb, pw, peps = 2, delta.y, delta.y_bias, delta.gate, delta.gate_bias, delta.weight, delta.eps
+            self._chk(y, None, (n, d), "branch output")
+            self._chk(g, y.dtype, (n, d), "gate")
+            for t, what in ((yb, "branch bias"), (gb, "gate bias"), (pw, "norm weight")):
+                if t is not None:
+                    self._chk(t, torch.float32, (d,), what)
+        elif delta is not None:
+            kind, y = 1, self._chk(delta, None, (n, d), "branch output")
+        if y is not None and y.dtype != out_dtype:
+            raise KernelError(f"branch output in {y.dtype}, rows wanted in {out_dtype}")
+        if weight is not None:
+            self._chk(weight, torch.float32, (d,), "norm weight")
+        x_out = torch.empty_like(x) if kind else None
+        h = torch.empty(n, d, dtype=out_dtype, device=x.device) if do_norm else None
+        hs = sw = state = None
+        rows = 1
+        if shift is not None:
+            sw, state = shift
+            self._chk(sw, torch.float32, (d,), "shift weight")
+            self._chk(state, torch.float32, (state.shape[0], 2, d), "shift state")
+            hs = torch.empty(n, d, dtype=out_dtype, device=x.device)
+            rows = self.SHIFT_ROWS_PER_BLOCK if n >= 4 * self._compute_units * self.SHIFT_ROWS_PER_BLOCK else 1
+        is_bf16 = 1 if out_dtype == torch.bfloat16 else 0
+        self._call("jle_add_norm_shift", _p(x), _p(x_out), kind, _p(y), _p(yb), _p(g), _p(gb), _p(pw), float(peps),
+                   int(do_norm), _p(weight), float(eps), _p(h), _p(sw), _p(hs), _p(state),
+                   _p(ctx.positions) if shift is not None else None,
+                   _p(ctx.token_segment) if shift is not None else None,
+                   _p(ctx.cu_seqlens) if shift is not None else None,
+                   _p(ctx.state_slots) if shift is not None else None,
+                   _p(ctx.state_phase) if shift is not None else None, is_bf16, n, d, rows)
+        return (x_out if kind else x), h, hs
+
+    def polynorm(self, z, bias, coef, eps: float):
+        """``c0 N(u) + c1 N(u^2) + c2 N(u^3) + c3`` with ``u = z + bias``, ``N`` a row's division by its root mean
+        square (float32 inside)."""
+        n, f = z.shape
+        self._chk(z, None, (n, f), "feed-forward rows")
+        self._chk(coef, torch.float32, (4,), "activation coefficients")
+        if bias is not None:
+            self._chk(bias, torch.float32, (f,), "bias")
+        out = torch.empty_like(z)
+        self._call("jle_polynorm", _p(z), f, _p(bias), _p(coef), float(eps), _p(out), self._is_bf16(z), n, f)
+        return out
+
+    def batched_linear(self, a, w, tokens_first: bool = False):
+        """``out[b] = a[b] @ w[b]`` for ``a [B, N, K]``, ``w [B, K, M]`` (views with any strides): a library
+        product, true float32 in float32.  ``[B, N, M]``, or with ``tokens_first`` laid out ``[N, B, M]``."""
+        out = torch.bmm(a, w)
+        return out.transpose(0, 1).contiguous() if tokens_first else out
+
+    def latent_prepare(self, rows, num_heads: int, nope_dim: int, rope_dim: int, kv_rank: int, positions, rotation,
+                       latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool) -> None:
+        n, ld = rows.shape
+        self._chk(rows, None, None, "projected rows")
+        self._chk(positions, torch.int32, (n,), "positions")
+        pairing, rd, inv = 0, 0, None
+        if rotation is not None:
+            rd = int(rotation.rotary_dim) or rope_dim
+            pairing = {"adjacent": 0, "half": 1}[rotation.pairing]
+            inv = self._chk(rotation.inv_freq, torch.float32, (rd // 2,), "rotary frequencies")
+        if writes:
+            np_, ps = latent_pages.shape[0], latent_pages.shape[1]
+            self._chk(latent_pages, rows.dtype, (np_, ps, kv_rank), "latent pages")
+            self._chk(rope_pages, rows.dtype, (np_, ps, rope_dim), "rotated key pages")
+            self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+            if latent_norm is not None:
+                self._chk(latent_norm, torch.float32, (kv_rank,), "latent norm weight")
+        self._call("jle_latent_prepare", _p(rows), ld, num_heads, nope_dim, rope_dim, kv_rank, _p(positions), _p(inv),
+                   pairing, rd, _p(latent_norm) if writes else None, float(eps),
+                   _p(latent_pages) if writes else None, _p(rope_pages) if writes else None,
+                   _p(slot_mapping) if writes else None, int(bool(writes)), self._is_bf16(rows), n)
+
+    LATENT_SPLIT_BELOW = 2048  # fewer (token, head) pairs than this: a query's key tiles are shared between wavefronts
+
+    def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
+                         token_segment, window, scale: float, meta=None):
+        """See ``attention_latent.hip``.  ``q_lat [H, N, kv_rank]``, ``q [N, H, nope + rope]`` (a view of the
+        projected rows: the heads' queries lie at their start); returns ``[N, H, kv_rank]``."""
+        H, n, r = q_lat.shape
+        dr = q.shape[2] - nope_dim
+        np_, ps = latent_pages.shape[0], latent_pages.shape[1]
+        self._chk(q_lat, latent_pages.dtype, (H, n, r), "queries in the latent's space")
+        if q.dtype != q_lat.dtype or q.stride(2) != 1 or q.stride(1) != q.shape[2] or q.shape[:2] != (n, H):
+            raise KernelError("the heads' queries must lie side by side at the start of contiguous rows")
+        q_ld = q.stride(0)  # (rows that also hold the latent: a token's queries are addressed by the row's full width)
+        self._chk(latent_pages, None, (np_, ps, r), "latent pages")
+        self._chk(rope_pages, latent_pages.dtype, (np_, ps, dr), "rotated key pages")
+        self._chk(block_table, torch.int32, None, "block table")
+        self._chk(positions, torch.int32, (n,), "positions")
+        self._chk(token_segment, torch.int32, (n,), "token segments")
+        w = 0 if window is None else int(window)
+        out = torch.empty(n, H, r, dtype=q_lat.dtype, device=q_lat.device)
+        splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
+        waves = n * H
+        if waves < self.LATENT_SPLIT_BELOW:
+            if meta is not None and meta.decode_bucket is not None:
+                longest = meta.decode_bucket  # (a step of single tokens: laid out for the bound, see GroupContext)
+            elif meta is not None and meta.seg_starts is not None:
+                longest = max(s0 + ln for s0, ln in zip(meta.seg_starts, meta.seg_lens))
+            else:
+                longest = int(positions.max()) + 1
+            span = min(w, longest) if w else longest
+            tiles = -(-span // 64) + 1
+            want = min(tiles, -(-self.LATENT_SPLIT_BELOW // waves))
+            if want > 1:
+                tiles_per_split = -(-tiles // want)
+                splits = -(-tiles // tiles_per_split)
+                ws_ml = torch.empty(waves * splits * 2, dtype=torch.float32, device=q.device)
+                ws_o = torch.empty(waves * splits * r, dtype=torch.float32, device=q.device)
+        self._call("jle_latent_attention", _p(q_lat), _p(q), q_ld, nope_dim, dr, _p(latent_pages), _p(rope_pages), _p(out),
+                   _p(positions), _p(token_segment), _p(block_table), block_table.shape[1], w, float(scale),
+                   self._is_bf16(q_lat), n, H, r, ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
+        return out
+
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
+        if hasattr(delta, "gate"):  # a gated branch: the kernel that knows it (the sum goes into a new array)
+            x_out, h, _ = self.add_norm_shift(x, delta, weight, eps, out_dtype, None, None)
+            x.copy_(x_out)
+            return h, (h.float() if want32 else None)
         n, d = x.shape
         self._chk(x, torch.float32, (n, d), "residual")
         kind, plain, routed, inv, k, shared, is_bf16 = 0, None, None, None, 0, None, 0
@@ -233,6 +370,10 @@ class HipOps:
         return out
 
     def add_residual(self, x, delta) -> None:
+        if hasattr(delta, "gate"):
+            x_out, _, _ = self.add_norm_shift(x, delta, None, 0.0, delta.y.dtype, None, None, do_norm=False)
+            x.copy_(x_out)
+            return
         delta = self.materialize(delta)
         self._chk(x, torch.float32, None, "residual")
         self._chk(delta, None, x.shape, "branch output")

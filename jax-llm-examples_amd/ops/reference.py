@@ -43,8 +43,44 @@ class ReferenceOps:
         return table[token_ids.long()].float()
 
     # ------------------------------------------------------------------ norms
+    def materialize(self, delta):
+        """The tensor a branch output that is not formed yet stands for (float32)."""
+        if hasattr(delta, "gate"):  # a GatedBranch: rmsnorm((y + b) * sigmoid(g + c)) * weight
+            t = delta.y.float() if delta.y_bias is None else delta.y.float() + delta.y_bias.float()
+            g = delta.gate.float() if delta.gate_bias is None else delta.gate.float() + delta.gate_bias.float()
+            t = t * torch.sigmoid(g)
+            t = t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + delta.eps)
+            return t if delta.weight is None else t * delta.weight.float()
+        return delta
+
+    def add_norm_shift(self, x, delta, weight, eps: float, out_dtype, shift, ctx):
+        """``x' = x + delta`` (a new tensor, float32; ``delta`` a tensor, a gated branch or ``None``), ``h =
+        rmsnorm(x') * weight`` and, with ``shift = (w, state)``, ``hs = h + (h_prev - h) * w`` where ``h_prev`` is
+        the float32 ``h`` of the token before: the row before in the same segment, or for a segment's first row
+        the request's state (``state[slot, phase]``; zeros at position 0).  The last row's ``h`` of every segment
+        goes into ``state[slot, 1 - phase]``.  Returns ``(x', h, hs or None)``."""
+        x = x if delta is None else x + self.materialize(delta).float()
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        if weight is not None:
+            h = h * weight.float()
+        hs = None
+        if shift is not None:
+            w, state = shift
+            prev = torch.empty_like(h)
+            prev[1:] = h[:-1]
+            cu = ctx.cu_seqlens.long()
+            first, last = cu[:-1], cu[1:] - 1
+            slots, phase = ctx.state_slots.long(), ctx.state_phase.long()
+            carried = state[slots, phase].float()
+            carried = torch.where((ctx.positions.long()[first] == 0)[:, None], torch.zeros_like(carried), carried)
+            prev[first] = carried
+            state[slots, 1 - phase] = h[last].to(state.dtype)
+            hs = (h + (prev - h) * w.float()).to(out_dtype)
+        return x, h.to(out_dtype), hs
+
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
         """``x += delta`` (in place, float32), then ``h = x / sqrt(mean(x^2) + eps) * weight``."""
+        delta = self.materialize(delta)
         if delta is not None:
             x.add_(delta.float())
         h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
@@ -53,7 +89,7 @@ class ReferenceOps:
         return h.to(out_dtype), (h if want32 else None)
 
     def add_residual(self, x, delta) -> None:
-        x.add_(delta.float())
+        x.add_(self.materialize(delta).float())
 
     def gather_rows(self, x, idx):
         return x[idx.long()]
@@ -70,13 +106,89 @@ class ReferenceOps:
     def swiglu_linear(self, h, w_gate_up):
         return self.silu_mul(self.linear(h, w_gate_up))
 
-    def materialize(self, delta):
-        return delta
-
     def silu_mul(self, gate_up):
         f = gate_up.shape[-1] // 2
         g, u = gate_up[..., :f].float(), gate_up[..., f:].float()
         return (torch.nn.functional.silu(g) * u).to(gate_up.dtype)
+
+    def batched_linear(self, a, w, tokens_first: bool = False):
+        """``out[b] = a[b] @ w[b]`` for ``a [B, N, K]`` and ``w [B, K, M]`` (views with any strides);
+        ``[B, N, M]``, or with ``tokens_first`` the same numbers laid out ``[N, B, M]``."""
+        out = torch.bmm(a.float(), w.float()).to(a.dtype)
+        return out.transpose(0, 1).contiguous() if tokens_first else out
+
+    def polynorm(self, z, bias, coef, eps: float):
+        """``c0 N(u) + c1 N(u^2) + c2 N(u^3) + c3`` with ``u = z + bias`` and ``N(v) = v / sqrt(mean(v^2) + eps)``
+        over a row, float32 inside."""
+        u = z.float() if bias is None else z.float() + bias.float()
+        n = lambda v: v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        c = coef.float()
+        return (c[0] * n(u) + c[1] * n(u * u) + c[2] * n(u * u * u) + c[3]).to(z.dtype)
+
+    # ------------------------------------------------------------------ attention over a cached latent
+    @staticmethod
+    def _turn(x, positions, rotation):
+        """The leading ``rotary_dim`` elements of the last axis turned by ``pos * inv_freq`` (float32 angles)."""
+        if rotation is None:
+            return x
+        rd = int(rotation.rotary_dim) or x.shape[-1]
+        ang = positions.float()[:, None] * rotation.inv_freq.float()[None, :]
+        sin, cos = torch.sin(ang), torch.cos(ang)
+        while sin.dim() < x.dim():
+            sin, cos = sin.unsqueeze(1), cos.unsqueeze(1)
+        head, rest = x[..., :rd], x[..., rd:]
+        if rotation.pairing == "adjacent":
+            pairs = head.reshape(*head.shape[:-1], rd // 2, 2)
+            a, b = pairs[..., 0], pairs[..., 1]
+            head = torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1).reshape(*head.shape[:-1], rd)
+        else:
+            a, b = head[..., : rd // 2], head[..., rd // 2:]
+            head = torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
+        return torch.cat([head, rest], dim=-1)
+
+    def latent_prepare(self, rows, num_heads: int, nope_dim: int, rope_dim: int, kv_rank: int, positions, rotation,
+                       latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool) -> None:
+        """``rows``: ``[N, H * (nope + rope) (+ kv_rank + rope)]``.  Turns the ``rope`` part of every head's
+        query in place; if the run writes its cache: RMS-norms the latent (the ``kv_rank`` numbers behind the
+        queries) with ``latent_norm``, turns the shared key part (the last ``rope`` numbers) and writes both
+        into their pages at ``slot = page * page_size + offset``."""
+        n = rows.shape[0]
+        H, dn, dr = num_heads, nope_dim, rope_dim
+        q = rows[:, : H * (dn + dr)].view(n, H, dn + dr)
+        q[:, :, dn:] = self._turn(q[:, :, dn:].float(), positions, rotation).to(rows.dtype)
+        if writes:
+            c = rows[:, H * (dn + dr): H * (dn + dr) + kv_rank].float()
+            c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps)
+            if latent_norm is not None:
+                c = c * latent_norm.float()
+            kr = self._turn(rows[:, H * (dn + dr) + kv_rank:].float(), positions, rotation)
+            ps = latent_pages.shape[1]
+            page, off = (slot_mapping // ps).long(), (slot_mapping % ps).long()
+            latent_pages[page, off] = c.to(latent_pages.dtype)
+            rope_pages[page, off] = kr.to(rope_pages.dtype)
+
+    def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
+                         token_segment, window, scale: float, meta=None):
+        """For every token and head: softmax over the visible cached tokens ``j`` (``0 <= pos - j < window``;
+        all earlier ones without a window) of ``(q_lat . c_j + q_r . k_j) * scale``, and the sum of the ``c_j``
+        with those weights.  ``q_lat``: ``[H, N, kv_rank]``; ``q``: ``[N, H, nope + rope]`` whose rotated part is
+        ``q_r``.  Returns ``[N, H, kv_rank]``."""
+        H, n, r = q_lat.shape
+        ps = latent_pages.shape[1]
+        out = torch.empty(n, H, r, dtype=q_lat.dtype, device=q_lat.device)
+        for i in range(n):
+            p = int(positions[i])
+            s = 0 if window is None else max(0, p - int(window) + 1)
+            kpos = torch.arange(s, p + 1, device=q_lat.device)
+            pages = block_table[int(token_segment[i])][(kpos // ps).long()].long()
+            if bool((pages < 0).any()):
+                raise RuntimeError(f"token {i} at position {p} reads a page that was given back")
+            off = (kpos % ps).long()
+            c = latent_pages[pages, off].float()  # [T, r]
+            kr = rope_pages[pages, off].float()  # [T, rope]
+            sc = (q_lat[:, i].float() @ c.t() + q[i, :, nope_dim:].float() @ kr.t()) * scale
+            out[i] = (torch.softmax(sc, dim=-1) @ c).to(out.dtype)
+        return out
 
     # ------------------------------------------------------------------ attention
     def qk_prepare_kv_write(self, qkv, num_heads: int, num_kv_heads: int, head_dim: int, positions, prep,

@@ -8,8 +8,11 @@ norm (or the end of the model) applies it.
 """
 from __future__ import annotations
 
+import torch
+
 from ..config.specs import LayerSpec
-from .base import build_feed_forward, build_mixer, build_norm
+from .base import ParamSpec, Part, build_feed_forward, build_mixer, build_norm
+from .residual import GatedBranch
 
 _ARRANGEMENTS = {}
 
@@ -56,3 +59,109 @@ class PreNormBlock:
         else:
             h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input)
         residual.add(ff.forward(h, h32, ctx))
+
+
+class SigmoidGate(Part):
+    """``sigmoid(W h + b)`` per element of a branch's output; this part holds ``W`` and ``b``, the kernel that
+    adds the branch to the residual applies the sigmoid and the product."""
+
+    graph_safe = True
+
+    def __init__(self, hidden: int) -> None:
+        super().__init__()
+        self.hidden = int(hidden)
+
+    def param_specs(self):
+        d = self.hidden
+        return {"weight": ParamSpec((d, d), init=("normal", d ** -0.5)),
+                "bias": ParamSpec((d,), policy="float32", init=("normal", 1.0))}
+
+    def forward(self, h, ctx):
+        """The gate before its sigmoid and without its bias: ``[N, hidden]`` in the run dtype."""
+        return ctx.ops.linear(h, self.params["weight"])
+
+
+class TokenShift(Part):
+    """``h + (h_prev - h) * weight`` per element, ``h_prev`` the row of the token before (zeros before a
+    sequence's first token).  The part holds the weight; the kernel that norms the rows does the mixing,
+    from a per-request state that carries the last row from step to step."""
+
+    graph_safe = True
+
+    def __init__(self, hidden: int) -> None:
+        super().__init__()
+        self.hidden = int(hidden)
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.hidden,), policy="float32", init=("uniform", 0.0, 1.0))}
+
+    def flops_per_token(self) -> float:
+        return 0.0
+
+
+@register_arrangement("sandwich_gated")
+class SandwichGatedBlock:
+    """A norm before and behind every branch, and a gate on its output::
+
+        h = norm(x);  x += post_norm(branch(h') * sigmoid(W_g h + b_g))
+
+    ``h'`` is ``h`` for the feed-forward and, with the option ``token_shift``, ``h`` mixed with the row of the
+    token before for the mixer (:class:`TokenShift`; the gate reads ``h`` itself).  The layer may have no
+    feed-forward.  The gated, normed branch output stays pending on the residual (a
+    :class:`~.residual.GatedBranch`); the kernel that forms the next norm's rows adds it first.
+    Options (``LayerSpec.options``): ``hidden_size``, ``post_norm`` (the spec of the two norms behind the
+    branches), ``token_shift``."""
+
+    def __init__(self, spec: LayerSpec) -> None:
+        self.spec = spec
+        opt = spec.options
+        d = int(opt["hidden_size"])
+        self.mixer = build_mixer(spec.mixer)
+        self.mixer_norm = build_norm(spec.mixer_norm)
+        self.mixer_post_norm = build_norm(opt["post_norm"])
+        self.mixer_gate = SigmoidGate(d)
+        self.token_shift = TokenShift(d) if opt.get("token_shift") else None
+        self.feed_forward = None
+        if spec.feed_forward is not None:
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+            self.feed_forward_post_norm = build_norm(opt["post_norm"])
+            self.feed_forward_gate = SigmoidGate(d)
+        self.hidden = d
+
+    def parts(self):
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm, "mixer_post_norm": self.mixer_post_norm,
+               "mixer_gate": self.mixer_gate}
+        if self.token_shift is not None:
+            out["token_shift"] = self.token_shift
+        if self.feed_forward is not None:
+            out.update(feed_forward=self.feed_forward, feed_forward_norm=self.feed_forward_norm,
+                       feed_forward_post_norm=self.feed_forward_post_norm, feed_forward_gate=self.feed_forward_gate)
+        return out
+
+    def run_state_need(self) -> dict:
+        """Per-request state of one run of this layer: the last token's normed row, for the shift."""
+        return {"shift": ((self.hidden,), torch.float32)} if self.token_shift is not None else {}
+
+    def forward(self, residual, ctx, cache) -> None:
+        shift = None
+        if self.token_shift is not None:
+            shift = (self.token_shift.params["weight"], cache.run_state["shift"])
+        h, hs = residual.normed_shifted(ctx, self.mixer_norm.params.get("weight"), self.mixer_norm.eps, shift)
+        gate = self.mixer_gate.forward(h, ctx)
+        y = self.mixer.forward(hs, ctx, cache)
+        post = self.mixer_post_norm
+        residual.add(GatedBranch(y, None, gate, self.mixer_gate.params["bias"], post.params.get("weight"), post.eps))
+        ff = self.feed_forward
+        if ff is None:
+            return
+        h, _ = residual.normed_shifted(ctx, self.feed_forward_norm.params.get("weight"), self.feed_forward_norm.eps,
+                                       None)
+        gate = self.feed_forward_gate.forward(h, ctx)
+        if hasattr(ff, "forward_unbiased"):  # (the bias of its last product is added by the kernel that gates it)
+            y, bias = ff.forward_unbiased(h, None, ctx)
+        else:
+            y, bias = ff.forward(h, None, ctx), None
+        post = self.feed_forward_post_norm
+        residual.add(GatedBranch(y, bias, gate, self.feed_forward_gate.params["bias"], post.params.get("weight"),
+                                 post.eps))

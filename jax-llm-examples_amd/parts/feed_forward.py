@@ -103,3 +103,39 @@ class MoESigmoidShared(FeedForward):
         shared = (self.params["shared_gate_up"], self.params["shared_down"]) if self.shared_inter else None
         return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"],
                                shared_weights=shared, tiled=self.tiled, grouping=grouping)
+
+
+@register_feed_forward("dense_polynorm")
+class DensePolyNorm(FeedForward):
+    """``W_down act(W_up h + b_up) + b_down`` with the polynomial activation
+    ``act(z) = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3``: powers element by element, ``N`` divides a token's row
+    by its root mean square (``eps`` inside the root; float32)."""
+
+    def __init__(self, spec) -> None:
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+        self.inter = int(spec.intermediate_size)
+        self.eps = float(spec.eps)
+
+    def param_specs(self):
+        d, f = self.hidden, self.inter
+        return {
+            "w_up": ParamSpec((f, d), init=("normal", d ** -0.5)),
+            "b_up": ParamSpec((f,), policy="float32", init=("normal", 0.1)),
+            "w_down": ParamSpec((d, f), init=("normal", f ** -0.5)),
+            "b_down": ParamSpec((d,), policy="float32", init=("normal", 0.1)),
+            "coef": ParamSpec((4,), policy="float32", init=("uniform", -1.0, 1.0)),
+        }
+
+    graph_safe = True
+
+    def forward_unbiased(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx):
+        """``(W_down act(...), b_down)``: for a caller whose next kernel adds the bias itself."""
+        ops = ctx.ops
+        z = ops.linear(h, self.params["w_up"])
+        a = ops.polynorm(z, self.params["b_up"], self.params["coef"], self.eps)
+        return ops.linear(a, self.params["w_down"]), self.params["b_down"]
+
+    def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
+        y, b = self.forward_unbiased(h, h32, ctx)
+        return (y.float() + b).to(y.dtype)

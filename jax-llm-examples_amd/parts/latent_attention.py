@@ -1,0 +1,107 @@
+"""Attention over a cached low-rank latent.
+
+A token leaves two things in the cache: a latent ``c`` (``kv_rank`` numbers, RMS-normed with a weight) and one
+rotated key part ``k_r`` (``rope_dim`` numbers) that all heads share.  A head's key is ``[W_uk c, k_r]``, its
+value ``W_uv c``; its query ``[q_n, q_r]`` (``nope_dim`` unrotated and ``rope_dim`` rotated numbers), and
+
+    score = (q_n . W_uk c + q_r . k_r) * softmax_scale.
+
+Neither keys nor values are ever formed.  ``q_n . W_uk c = (W_uk^T q_n) . c``, so the query is taken into the
+latent's space (one batched product per step), the attention kernel runs over the cached ``[c, k_r]`` rows
+with all heads sharing them and sums the latents with the softmax weights, and ``W_uv`` is applied to that sum
+(a second batched product).  Prefill and decode are the same computation, so a token's result does not depend
+on how its request was cut into steps.
+
+Options as data: ``window`` (a query sees itself and the ``window - 1`` tokens before it; ``None``: all),
+``retention`` (what the cache keeps: at least the window of every run that reads it), ``own_latent`` (False: the
+run projects no latent and reads a cache that another run writes), ``position`` (a rotary kind for ``q_r`` and
+``k_r``), ``latent_norm_eps``.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import CacheNeed, Mixer, ParamSpec, build_position, register_mixer
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    def __init__(self, spec) -> None:
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+        self.num_heads = int(spec.num_heads)
+        self.nope_dim, self.rope_dim = int(spec.nope_dim), int(spec.rope_dim)
+        self.value_dim, self.kv_rank = int(spec.value_dim), int(spec.kv_rank)
+        self.softmax_scale = float(spec.softmax_scale)
+        w = spec.get("window")
+        self.window = None if w is None else int(w)
+        self.retention = tuple(spec.get("retention") or (("all",) if self.window is None else ("window", self.window)))
+        if self.retention[0] == "window" and (self.window is None or self.window > int(self.retention[1])):
+            raise ValueError(f"the cache keeps {self.retention}, less than the window {self.window} of a run that reads it")
+        if self.retention[0] not in ("all", "window"):
+            raise ValueError(f"the latent attention reads its cache under 'all' or 'window', not {self.retention!r}")
+        self.own_latent = bool(spec.get("own_latent", True))
+        self.latent_norm_eps = float(spec.latent_norm_eps)
+        self.position = build_position(spec.position, self.rope_dim)
+        self.rotation = None
+
+    @property
+    def q_rows(self) -> int:
+        return self.num_heads * (self.nope_dim + self.rope_dim)
+
+    def param_specs(self):
+        h, d = self.num_heads, self.hidden
+        kv = self.kv_rank + self.rope_dim if self.own_latent else 0
+        specs = {
+            # rows: the heads' queries ([unrotated, rotated] per head), then the latent, then the shared rotated key
+            "w_in": ParamSpec((self.q_rows + kv, d), init=("normal", d ** -0.5)),
+            "w_uk": ParamSpec((h * self.nope_dim, self.kv_rank), init=("normal", self.kv_rank ** -0.5)),
+            "w_uv": ParamSpec((h * self.value_dim, self.kv_rank), init=("normal", self.kv_rank ** -0.5)),
+            "wo": ParamSpec((d, h * self.value_dim), init=("normal", (h * self.value_dim) ** -0.5)),
+        }
+        if self.own_latent:
+            specs["latent_norm"] = ParamSpec((self.kv_rank,), policy="float32", init=("uniform", 0.5, 1.5))
+        return specs
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(paged=(("latent", (self.kv_rank,)), ("rope_key", (self.rope_dim,))), retention=self.retention)
+
+    graph_safe = True
+
+    def finalize(self) -> None:
+        rot = self.position.rotation()
+        if rot is not None:
+            rot.inv_freq = rot.inv_freq.to(self.params["w_in"].device)
+        self.rotation = rot
+
+    def mixing_flops(self, start: int, count: int) -> float:
+        """Scores and sums over the visible latents, and the two batched products that take queries into the
+        latent's space and the sums out of it."""
+        w = self.window
+        keys = sum(min(p + 1, w) if w is not None else p + 1 for p in range(start, start + count))
+        h, r = self.num_heads, self.kv_rank
+        return (2.0 * h * (2 * r + self.rope_dim) * keys + 2.0 * count * h * r * (self.nope_dim + self.value_dim))
+
+    def flops_per_token(self) -> float:
+        return 2.0 * (self.params["w_in"].numel() + self.params["wo"].numel())
+
+    def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
+        ops = ctx.ops
+        H, dn, dr, dv, r = self.num_heads, self.nope_dim, self.rope_dim, self.value_dim, self.kv_rank
+        n = h.shape[0]
+        rows = ops.linear(h, self.params["w_in"])  # [N, H * (dn + dr) (+ r + dr)]
+        if self.own_latent != bool(cache.writes):
+            raise ValueError("a run with a latent of its own writes its cache, one without reads another's")
+        # rotates q_r in place, norms the latent, rotates the shared key part and writes both into their pages
+        ops.latent_prepare(rows, H, dn, dr, r, ctx.positions, self.rotation,
+                           self.params.get("latent_norm"), self.latent_norm_eps,
+                           cache.pages["latent"], cache.pages["rope_key"], cache.slot_mapping, cache.writes)
+        q = rows[:, : self.q_rows].view(n, H, dn + dr)
+        # queries into the latent's space: [H, N, dn] x [H, dn, r]
+        q_lat = ops.batched_linear(q[:, :, :dn].transpose(0, 1), self.params["w_uk"].view(H, dn, r))
+        o_lat = ops.latent_attention(q_lat, q, dn, cache.pages["latent"], cache.pages["rope_key"], cache.block_table,
+                                     ctx.positions, ctx.token_segment, self.window, self.softmax_scale,
+                                     cache.attn_meta)  # [N, H, r]
+        # the sums out of it: [H, N, r] x [H, r, dv], laid out [N, H * dv]
+        o = ops.batched_linear(o_lat.transpose(0, 1), self.params["w_uv"].view(H, dv, r).transpose(1, 2), tokens_first=True)
+        return ops.linear(o.view(n, H * dv), self.params["wo"])

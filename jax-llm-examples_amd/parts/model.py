@@ -74,15 +74,27 @@ class DecoderModel:
             needs[e.cache] = need
         return needs
 
+    def run_state_needs(self) -> dict[int, dict]:
+        """Fixed-size per-request state that the arrangements keep, by place in the run order (every run has its
+        own, also a run that reads another run's cache): ``{name: (shape, dtype)}``."""
+        out: dict[int, dict] = {}
+        for k, e in enumerate(self.plan.order):
+            need = getattr(self.blocks[e.layer], "run_state_need", None)
+            need = need() if need is not None else {}
+            if need:
+                out[k] = dict(need)
+        return out
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, cache) -> torch.Tensor:
         """Runs the step's tokens through every run of the order; returns float32
         logits ``[len(ctx.logits_indices), vocab]``."""
         ops = ctx.ops
         residual = Residual(self.embed.forward(ctx.token_ids, ctx))
-        for e in self.plan.order:
+        for k, e in enumerate(self.plan.order):
             gi = cache.group_of.get(e.cache)
-            view = CacheView(cache_id=e.cache, writes=e.writes_cache, group=gi, state=cache.state.get(e.cache))
+            view = CacheView(cache_id=e.cache, writes=e.writes_cache, group=gi, state=cache.state.get(e.cache),
+                             run_state=cache.run_state.get(k))
             if gi is not None:
                 g = ctx.groups[gi]
                 view.kv = cache.groups[gi].tensors.get(e.cache)
@@ -91,6 +103,8 @@ class DecoderModel:
                 view.slot_mapping = g.slot_mapping
                 view.attn_meta = g
             self.blocks[e.layer].forward(residual, ctx, view)
+            if ctx.tap is not None:  # (whoever watches the step sees the residual stream behind every run)
+                ctx.tap(self.blocks[e.layer], "residual", lambda r=residual: r.value(ctx).clone())
         if ctx.logits_indices.numel() == 0:
             residual.value(ctx)
             return torch.empty(0, self.plan.vocab_size, dtype=torch.float32, device=ctx.device)

@@ -60,3 +60,19 @@ class RopeInterleaved(PositionEncoding):
 
     def rotation(self) -> Rotation:
         return Rotation(self.inv_freq(), pairing="adjacent", rotary_dim=self.head_dim)
+
+
+@register_position("rope_half")
+class RopeHalf(PositionEncoding):
+    """Rotary embedding over half-split pairs: element ``j`` pairs with ``j + rotary_dim / 2`` for ``j`` below
+    ``rotary_dim / 2``; the pair ``(u, v)`` at position ``p`` becomes ``(u cos a - v sin a, v cos a + u sin a)``
+    with ``a = p * theta ** (-2 j / rotary_dim)``.  ``rotary_dim`` leading elements of the vector turn (default:
+    all), the rest pass unchanged."""
+
+    def rotation(self) -> Rotation:
+        rd = int(self.spec.get("rotary_dim") or self.head_dim)
+        if rd % 2 or not 0 < rd <= self.head_dim:
+            raise ValueError(f"rotary_dim must be even and at most {self.head_dim}, got {rd}")
+        j = torch.arange(0, rd // 2, dtype=torch.float64)
+        inv = torch.tensor(float(self.spec.theta), dtype=torch.float64) ** (-2.0 * j / rd)
+        return Rotation(inv.to(torch.float32), pairing="half", rotary_dim=rd)

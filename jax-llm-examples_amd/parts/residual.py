@@ -6,6 +6,21 @@ from __future__ import annotations
 import torch
 
 
+class GatedBranch:
+    """A branch output that is not formed yet: ``rmsnorm((y + y_bias) * sigmoid(gate + gate_bias)) * weight``
+    per row (statistics over the row, ``eps`` inside the root, float32).  ``y`` and ``gate`` are ``[N, hidden]``
+    in the run dtype, the biases and the weight float32 ``[hidden]`` or ``None``.  The kernel that adds it to
+    the residual reads the pieces directly."""
+
+    def __init__(self, y, y_bias, gate, gate_bias, weight, eps: float) -> None:
+        self.y, self.y_bias, self.gate, self.gate_bias, self.weight, self.eps = y, y_bias, gate, gate_bias, weight, float(eps)
+        self.shape, self.dtype = y.shape, y.dtype
+
+    def rows(self, ops, idx) -> "GatedBranch":
+        return GatedBranch(ops.gather_rows(self.y, idx), self.y_bias, ops.gather_rows(self.gate, idx),
+                           self.gate_bias, self.weight, self.eps)
+
+
 class Residual:
     def __init__(self, x: torch.Tensor) -> None:
         assert x.dtype == torch.float32
@@ -19,7 +34,7 @@ class Residual:
             self._x, self._deferred = self._deferred.residual(), None
         return self._x
 
-    def add(self, delta: torch.Tensor) -> None:
+    def add(self, delta) -> None:
         if self.pending is not None:
             raise AssertionError("a branch output is already pending on the residual")
         if delta.shape != self.x.shape:
@@ -37,6 +52,16 @@ class Residual:
         self.pending = None
         return h, h32
 
+    def normed_shifted(self, ctx, weight, eps: float, shift=None):
+        """Adds what is pending, norms the rows and, with ``shift = (weight, state)``, also gives the rows mixed
+        with the rows of the tokens before them (see :class:`~.block.TokenShift`; ``state``: float32
+        ``[slots, 2, hidden]``, the last row of every request, one half read and the other written by a
+        step).  The addition is not done in place: a row's kernel forms the row before it anew.  Returns
+        ``(h, shifted h or None)`` in the run dtype."""
+        self._x, h, hs = ctx.ops.add_norm_shift(self.x, self.pending, weight, eps, ctx.dtype, shift, ctx)
+        self.pending = None
+        return h, hs
+
     def value(self, ctx) -> torch.Tensor:
         if self.pending is not None:
             ctx.ops.add_residual(self.x, self.pending)
@@ -47,5 +72,8 @@ class Residual:
         """The residual of the chosen rows only (what is pending stays pending)."""
         r = Residual(ctx.ops.gather_rows(self.x, idx))
         if self.pending is not None:
-            r.pending = ctx.ops.gather_rows(self.pending, idx)
+            if hasattr(self.pending, "rows"):
+                r.pending = self.pending.rows(ctx.ops, idx)
+            else:
+                r.pending = ctx.ops.gather_rows(self.pending, idx)
         return r

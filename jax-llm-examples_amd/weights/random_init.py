@@ -2,7 +2,7 @@
 
 ``write_random_model`` writes a model folder (``config.json`` and
 ``model.safetensors`` with the checkpoint's own tensor names and layouts) from a
-configuration and a seed: every matrix N(0, 0.02), norm weights 1.  Each
+configuration and a seed: every tensor drawn as its binding says (``init``: N(0, std), uniform, or ones).  Each
 tensor's generator is seeded from ``(seed, tensor name)``, so a tensor's values
 do not depend on which others exist or in which order they are drawn.  (The
 reference draws one key per leaf by splitting one key in pytree order,
@@ -34,6 +34,10 @@ def draw(b: TensorBinding, seed: int, dtype: torch.dtype) -> torch.Tensor:
     if b.init[0] == "normal":
         g = torch.Generator().manual_seed(_seed_for(seed, b.name))
         return (torch.randn(b.shape, generator=g, dtype=torch.float32) * float(b.init[1])).to(dtype)
+    if b.init[0] == "uniform":
+        g = torch.Generator().manual_seed(_seed_for(seed, b.name))
+        lo, hi = float(b.init[1]), float(b.init[2])
+        return (torch.rand(b.shape, generator=g, dtype=torch.float32) * (hi - lo) + lo).to(dtype)
     raise ValueError(f"unknown init {b.init!r}")
 
 
@@ -67,6 +71,10 @@ def init_random_(model, seed: int, std: float = 0.02) -> None:
             t.fill_(1.0)
             continue
         g = torch.Generator(device=t.device).manual_seed(_seed_for(seed, name))
+        if init[0] == "uniform":
+            lo, hi = float(init[1]), float(init[2])
+            t.copy_(torch.rand(t.shape, generator=g, dtype=torch.float32, device=t.device) * (hi - lo) + lo)
+            continue
         s = float(init[1]) if init[0] == "normal" else std
         flat = t.view(-1)
         step = 1 << 28  # draw in pieces: no float32 copy of a whole large tensor
