@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     const T* __restrict__ latent_pages, const T* __restrict__ rope_pages, T* __restrict__ out /* [N, H, R] */,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, int window, float scale, int N, int H, int R, int ps, int splits, int tiles_per_split,
-    float* __restrict__ ws_ml, float* __restrict__ ws_o) {
+    float* __restrict__ ws_ml, float* __restrict__ ws_o, int vec /* rows may be read 16 bytes at a time */) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= N * H * splits) return;  // whole wavefront leaves; no block-wide barrier below
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
         const T* krow = rope_pages + slot * dr;
         float dot = 0.f;
         int c = 0;
-        for (; c + Vec16L<T>::kN <= R; c += Vec16L<T>::kN) {
+        for (; vec && c + Vec16L<T>::kN <= R; c += Vec16L<T>::kN) {
           Vec16L<T> a, b;
           a.load(ql + c);
           b.load(crow + c);
@@ -279,9 +279,9 @@ JLE_API int jle_latent_attention(const void* q_lat, const void* q, int q_ld, int
                                  hipStream_t s) {
   if (N <= 0) return 0;
   if (q_ld < H * (dn + dr) || H <= 0 || R <= 0 || R > 64 * kMaxAcc || dr <= 0 || dn < 0 || ps <= 0 || window < 0) return JLE_BAD_ARG;
-  // rows are read 16 bytes at a time
+  // rows are read 16 bytes at a time where every row starts at a multiple of 16 bytes
   const int per16 = is_bf16 ? 8 : 4;
-  if (R % per16) return JLE_BAD_ARG;
+  const int vec = R % per16 == 0 && (uintptr_t)q_lat % 16 == 0 && (uintptr_t)latent_pages % 16 == 0;
   if (splits < 1 || (splits > 1 && (tiles_per_split < 1 || ws_ml == nullptr || ws_o == nullptr))) return JLE_BAD_ARG;
   const long long items = (long long)N * H * splits;
   if (items > (1ll << 31) - 8) return JLE_BAD_ARG;
@@ -290,7 +290,7 @@ JLE_API int jle_latent_attention(const void* q_lat, const void* q, int q_ld, int
   if (is_bf16) {
     hipLaunchKernelGGL(latent_attention_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)q_lat, (const bf16_t*)q, q_ld, dn, dr,
                        (const bf16_t*)latent_pages, (const bf16_t*)rope_pages, (bf16_t*)out, positions, token_segment,
-                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o);
+                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o, vec);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(latent_attention_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * H, R,
@@ -298,7 +298,7 @@ JLE_API int jle_latent_attention(const void* q_lat, const void* q, int q_ld, int
   } else {
     hipLaunchKernelGGL(latent_attention_kernel<float>, g, b, 0, s, (const float*)q_lat, (const float*)q, q_ld, dn, dr,
                        (const float*)latent_pages, (const float*)rope_pages, (float*)out, positions, token_segment,
-                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o);
+                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o, vec);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(latent_attention_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, N * H, R,
