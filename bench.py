@@ -26,6 +26,119 @@ PEAK_HBM_GBS = 8000.0  # MI355X: HBM3E 8 TB/s
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}  # dense MFMA
 
 
+# Layer sizes for --designs: width, heads, feed-forward width, the window (Rovidra) or chunk (Llama 4) of the
+# attention, and Rovidra's latent: unrotated / rotated query elements, value elements, latent width.
+DESIGN_SIZES = {
+    "2k": dict(width=2048, heads=16, ff=8192, span=1024, dim=128, rot=64, vdim=128, rank=512, vocab=32000),
+    "4k": dict(width=4096, heads=32, ff=14336, span=4096, dim=128, rot=64, vdim=128, rank=512, vocab=32000),
+    "5k": dict(width=5120, heads=40, ff=16384, span=4096, dim=128, rot=64, vdim=128, rank=512, vocab=32000),
+}
+
+
+def design_configs(size: dict, layers: int):
+    """config.json of a Rovidra model (every second layer reads the latent of the layer before it) and of the
+    closest model the engine has: Llama 4 with dense layers only, rotary chunked attention, equal sizes."""
+    mixer = {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot"], "vdim": size["vdim"],
+             "kv_rank": size["rank"], "scale": (size["dim"] + size["rot"]) ** -0.5,
+             "rot": {"base": 500000.0, "dims": size["rot"]}, "mask": {"size": size["span"]}}
+    rovidra = {"architecture": "Rovidra", "vocab": size["vocab"], "width": size["width"],
+               "embedding": {"scale": size["width"] ** 0.5}, "norm": {"eps": 1e-5},
+               "layers": [{"type": "latent_attention", "mixer": dict(mixer, **({"kv_from": i - 1} if i % 2 else {})),
+                           "mlp": {"kind": "dense", "ff": size["ff"]}} for i in range(layers)]}
+    llama = {"architectures": ["Llama4ForCausalLM"], "num_hidden_layers": layers, "hidden_size": size["width"],
+             "num_attention_heads": size["heads"], "num_key_value_heads": 8, "head_dim": 128,
+             "interleave_moe_layer_step": 1, "moe_layers": [], "num_local_experts": 1, "num_experts_per_tok": 1,
+             "intermediate_size": size["ff"], "intermediate_size_mlp": size["ff"], "vocab_size": size["vocab"],
+             "rope_theta": 500000.0, "rope_scaling": None, "no_rope_layers": [1] * layers,
+             "attention_chunk_size": size["span"], "use_qk_norm": True, "attn_temperature_tuning": False,
+             "rms_norm_eps": 1e-5, "tie_word_embeddings": False}
+    return {"rovidra": rovidra, "llama4-dense": llama}
+
+
+def bench_designs(args) -> int:
+    import torch
+
+    from jax_llm_examples_amd.cache import CacheManager
+    from jax_llm_examples_amd.config.registry import architecture_name, get_architecture
+    from jax_llm_examples_amd.engine import ModelRunner, StepEntry, get_ops, random_model
+    from jax_llm_examples_amd.engine.accounting import decode_step_bytes, prefill_flops
+
+    dev, page = "cuda:0", 16
+    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+    layers = args.layers or 4
+    names = list(DESIGN_SIZES) if args.designs == "all" else args.designs.split(",")
+    points_at = [(int(b), int(c)) for b, _, c in (spec.partition("@") for spec in args.design_points.split(","))]
+    T = args.prefill_tokens
+    ops = get_ops(dev)
+    out = {}
+    for size_name in names:
+        size = DESIGN_SIZES[size_name]
+        for design, top in design_configs(size, layers).items():
+            arch = get_architecture(architecture_name(top))
+            cfg = arch.parse_config(top)
+            model = random_model(arch, cfg, seed=0, dtype=args.dtype, device=dev)
+            need = max(b * (c + page) for b, c in points_at) + T + 4 * page
+            cache = CacheManager(model.cache_needs(), page_size=page, num_pages=-(-need // page),
+                                 max_requests=max(b for b, _ in points_at) + 1, dtype=model.dtype, device=dev,
+                                 run_states=model.run_state_needs())
+            for g in cache.groups:  # stand-in contents for contexts that are not computed
+                for t in list(g.tensors.values()) + [t for named in g.pages.values() for t in named.values()]:
+                    t.normal_(0.0, 0.5)
+            runner = ModelRunner(model, cache, ops)
+            gen = torch.Generator().manual_seed(0)
+            V = model.plan.vocab_size
+            res = {}
+            times = []
+            for it in range(3):
+                toks = torch.randint(0, V, (T,), generator=gen).tolist()
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                runner.step([StepEntry(f"p{it}", toks, [T - 1])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t1)
+                runner.finish(f"p{it}")
+            sec = min(times[1:])
+            res[f"prefill_{T}_tok_s"] = round(T / sec, 1)
+            res[f"prefill_{T}_mfma_frac"] = round(prefill_flops(model, T) / sec / PEAK_FLOPS[dkey], 4)
+            for b, c in points_at:
+                steps, warmup = args.point_steps, 3
+                ids = [f"d{b}_{c}_{i}" for i in range(b)]
+                for rid in ids:
+                    cache.add_request(rid)
+                    cache.reserve(rid, c - steps - warmup)
+                    cache.commit(rid)
+                last = torch.randint(0, V, (b,), generator=gen).tolist()
+
+                def one():
+                    nonlocal last
+                    logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(ids, last)])
+                    last = logits.argmax(dim=-1).tolist()
+
+                for _ in range(warmup):
+                    one()
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                for _ in range(steps):
+                    one()
+                torch.cuda.synchronize()
+                sec = (time.perf_counter() - t1) / steps
+                nb = decode_step_bytes(model, cache, [cache.num_tokens(r) for r in ids])
+                for rid in ids:
+                    runner.finish(rid)
+                res[f"decode_b{b}_c{c}_tok_s"] = round(b / sec, 1)
+                res[f"decode_b{b}_c{c}_ms"] = round(sec * 1e3, 3)
+                res[f"decode_b{b}_c{c}_hbm_frac"] = round(nb["total"] / sec / 1e9 / PEAK_HBM_GBS, 4)
+            print(f"[bench] {size_name} {design} ({layers} layers, {model.num_parameters() / 1e9:.2f} B parameters): {res}",
+                  file=sys.stderr, flush=True)
+            out[f"{size_name}/{design}"] = res
+            del runner, cache, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prefill and decode tok/s of two designs at equal layer sizes, random weights",
+                      "dtype": dkey, "n_gpus": 1, "layers": layers, "sizes": {n: DESIGN_SIZES[n] for n in names},
+                      "designs": out}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -44,7 +157,13 @@ def main() -> int:
                     "+ output tokens @ decode batch), comma-separated: tokens a second end to end")
     ap.add_argument("--preset", default="llama4-scout")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--design-points", default="1@2048,8@2048,64@2048", help="decode steps of --designs: batch@context")
+    ap.add_argument("--designs", default="", help="instead of the default workload: prefill and decode of the Rovidra "
+                    "design beside the dense Llama 4 layer of equal sizes, at the named sizes (comma-separated, of "
+                    + ", ".join(DESIGN_SIZES) + "; 'all')")
     args = ap.parse_args()
+    if args.designs:
+        return bench_designs(args)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus > 1 is not supported")
         return 2

@@ -54,6 +54,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ row
                                                              const float* __restrict__ inv_freq, int pairing, int rd,
                                                              const float* __restrict__ norm_w, float eps,
                                                              T* __restrict__ latent_pages, T* __restrict__ rope_pages,
+                                                             T* __restrict__ latent_t_pages, int ps,
                                                              const int* __restrict__ slot_mapping, int writes) {
   __shared__ float red[4];
   const size_t n = blockIdx.x;
@@ -88,6 +89,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ row
     float v = Num<T>::load(c + d) * inv;
     if (norm_w != nullptr) v *= norm_w[d];
     Num<T>::store(lp + d, v);
+    // the same numbers with the page's tokens as the fastest index, for the matrix-core kernel's second product
+    if (latent_t_pages != nullptr) Num<T>::store(latent_t_pages + ((slot / ps) * R + d) * ps + slot % ps, v);
   }
   T* rp = rope_pages + slot * dr;
   for (int j = threadIdx.x; j < half; j += 256) {
@@ -247,25 +250,235 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float
   }
 }
 
+
+// ------------------------------------------------------------------ on the matrix cores (bfloat16)
+// A wavefront takes 16 consecutive (token, head) rows of one segment (in token-major order: with 16 or more heads
+// they are heads of one token, with fewer the heads of a few neighbouring tokens) and walks their keys in steps of
+// 32 absolute positions.  Everything is transposed so that no operand is shuffled between the two products:
+//     S^T [key, row] = [c_key, k_r_key] . [q_lat_row, q_r_row]     (A: a key's row from its page, B: the queries, held)
+//     O^T [d, row]  += c^T [d, key] P^T [key, row]                 (A: the latent's transposed copy, B: P as S left it)
+// The first product's key rows are dealt so that a lane ends up with the probabilities of eight consecutive keys,
+// which is what the second product's B operand wants.  Softmax statistics in float32; a row's masks are its own
+// token's position and window.  With few rows the steps are shared between wavefronts and merged.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+__device__ __forceinline__ u32x4 load16(const bf16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+template <int NR>  // chunks of 32 latent elements: kv_rank <= 32 * NR
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ q, int q_ld, int dn, int dr,
+    const bf16_t* __restrict__ latent, const bf16_t* __restrict__ latent_t, const bf16_t* __restrict__ rope,
+    bf16_t* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_segment,
+    const int* __restrict__ block_table, int table_width, int window, float scale, const int* __restrict__ tiles,
+    int num_tiles, int N, int H, int R, int ps, int splits, int steps_per_split, float* __restrict__ ws_ml,
+    float* __restrict__ ws_o) {
+  const int lane = threadIdx.x & 63, g = lane >> 4, r = lane & 15;
+  const int item = blockIdx.x * 4 + wave_index();
+  if (item >= num_tiles * splits) return;  // whole wavefront leaves; no block-wide barrier below
+  const int tile = item / splits, sp = item - tile * splits;
+  const int row0 = tiles[2 * tile], nrows = tiles[2 * tile + 1];
+  const bool row_ok = r < nrows;
+  const int row = row0 + (row_ok ? r : 0);
+  const int n = row / H, h = row - n * H;
+  const int pos = positions[n];
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  const int* table = block_table + (size_t)token_segment[__builtin_amdgcn_readfirstlane(row0 / H)] * table_width;
+  int lo = row_ok ? first : 0x7fffffff, hi = row_ok ? pos : -1;
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) {
+    lo = min(lo, __shfl_xor(lo, o, 64));
+    hi = max(hi, __shfl_xor(hi, o, 64));
+  }
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  // the queries: B operands, column = this lane's row, 8 consecutive k per lane
+  bf16x8 qb[NR + 2];
+  {
+    const bf16_t* ql = q_lat + ((size_t)h * N + n) * R;
+#pragma unroll
+    for (int c = 0; c < NR; ++c) {
+      const int k0 = c * 32 + g * 8;
+      qb[c] = __builtin_bit_cast(bf16x8, k0 < R ? load16(ql + k0) : zero4);
+    }
+    const bf16_t* qr = q + (size_t)n * q_ld + (size_t)h * (dn + dr) + dn;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int k0 = c * 32 + g * 8;
+      qb[NR + c] = __builtin_bit_cast(bf16x8, k0 < dr ? load16(qr + k0) : zero4);
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[NR * 2];
+#pragma unroll
+  for (int dt = 0; dt < NR * 2; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int t_lo = (lo / 32) * 32, t_hi = hi;
+  if (splits > 1) {
+    t_lo += sp * steps_per_split * 32;
+    t_hi = min(hi, t_lo + steps_per_split * 32 - 1);
+  }
+  for (int t0 = t_lo; t0 <= t_hi; t0 += 32) {
+    f32x4 st[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int key = t0 + 8 * (r >> 2) + 4 * t + (r & 3);  // which key is row r of this A operand
+      const int page = key <= hi ? table[key / ps] : -1;
+      const bool have = page >= 0;
+      const size_t slot = have ? (size_t)page * ps + key % ps : 0;
+      const bf16_t* crow = latent + slot * R;
+      const bf16_t* krow = rope + slot * dr;
+#pragma unroll
+      for (int c = 0; c < NR; ++c) {
+        if (c * 32 < R) {
+          const int k0 = c * 32 + g * 8;
+          const bf16x8 a = __builtin_bit_cast(bf16x8, (have && k0 < R) ? load16(crow + k0) : zero4);
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[c], st[t], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        if (c * 32 < dr) {
+          const int k0 = c * 32 + g * 8;
+          const bf16x8 a = __builtin_bit_cast(bf16x8, (have && k0 < dr) ? load16(krow + k0) : zero4);
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[NR + c], st[t], 0, 0, 0);
+        }
+      }
+    }
+    // this lane now holds, for its row, the scores of keys t0 + 8 g .. + 7
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = t0 + 8 * g + e;
+      const bool ok = row_ok && key >= first && key <= pos;
+      sv[e] = ok ? st[e >> 2][e & 3] * scale : -INFINITY;
+      mx = fmaxf(mx, sv[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float p[8];
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+      psum += p[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+    const u32x4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+    const bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
+    // the latent's transposed copy: row d of a page holds its tokens side by side
+    const int key0 = t0 + 8 * g;
+    const int vpage = key0 <= hi ? table[key0 / ps] : -1;
+    const bf16_t* vbase = latent_t + ((size_t)(vpage < 0 ? 0 : vpage) * R + r) * ps + key0 % ps;
+    // tokens behind the rows' last position are not written yet: what lies there must not meet a zero weight
+    const int n_ok = min(8, hi - key0 + 1);
+    u32x4 keep;
+#pragma unroll
+    for (int w2 = 0; w2 < 4; ++w2)
+      keep[w2] = n_ok >= 2 * w2 + 2 ? 0xffffffffu : (n_ok == 2 * w2 + 1 ? 0x0000ffffu : 0u);
+#pragma unroll
+    for (int dt = 0; dt < NR * 2; ++dt) {
+      if (dt * 16 < R) {
+        u32x4 v = vpage >= 0 ? load16(vbase + (size_t)dt * 16 * ps) : zero4;
+        v &= keep;
+        acc[dt] *= corr;
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, acc[dt], 0, 0, 0);
+      }
+    }
+  }
+  if (!row_ok) return;
+  if (splits > 1) {
+    const size_t slot = (size_t)row * splits + sp;
+    if (g == 0) {
+      ws_ml[slot * 2] = m;
+      ws_ml[slot * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NR * 2; ++dt)
+      if (dt * 16 < R) *reinterpret_cast<f32x4*>(ws_o + slot * R + dt * 16 + g * 4) = acc[dt];
+    return;
+  }
+  const float inv = 1.0f / l;
+  bf16_t* o = out + (size_t)row * R;
+#pragma unroll
+  for (int dt = 0; dt < NR * 2; ++dt) {
+    if (dt * 16 < R) {
+      const uint2 w = {pack_bf16(acc[dt][0] * inv, acc[dt][1] * inv), pack_bf16(acc[dt][2] * inv, acc[dt][3] * inv)};
+      *reinterpret_cast<uint2*>(o + dt * 16 + g * 4) = w;
+    }
+  }
+}
+
 }  // namespace
+
+// Whether the matrix-core kernel takes these sizes (bfloat16 only): rows read 16 bytes at a time.
+JLE_API int jle_latent_attention_mfma_supported(int R, int dn, int dr, int q_ld, int ps) {
+  return R > 0 && R % 32 == 0 && R <= 512 && dr > 0 && dr % 8 == 0 && dr <= 64 && dn % 8 == 0 && q_ld % 8 == 0 &&
+         ps % 8 == 0;
+}
+
+// tiles: (first row, rows) pairs, rows = token * H + head, up to 16 rows of one segment each.  splits > 1: a tile's
+// steps of 32 keys are shared between `splits` wavefronts, steps_per_split each, and merged (ws as below).
+JLE_API int jle_latent_attention_mfma(const void* q_lat, const void* q, int q_ld, int dn, int dr,
+                                      const void* latent_pages, const void* latent_t_pages, const void* rope_pages,
+                                      void* out, const int* positions, const int* token_segment,
+                                      const int* block_table, int table_width, int window, float scale,
+                                      const int* tiles, int num_tiles, int N, int H, int R, int ps, int splits,
+                                      int steps_per_split, float* ws_ml, float* ws_o, hipStream_t s) {
+  if (N <= 0 || num_tiles <= 0) return 0;
+  if (!jle_latent_attention_mfma_supported(R, dn, dr, q_ld, ps) || H <= 0 || window < 0 || tiles == nullptr ||
+      latent_t_pages == nullptr || q_ld < H * (dn + dr))
+    return JLE_BAD_ARG;
+  if (splits < 1 || (splits > 1 && (steps_per_split < 1 || ws_ml == nullptr || ws_o == nullptr))) return JLE_BAD_ARG;
+  const long long items = (long long)num_tiles * splits;
+  if (items > (1ll << 31) - 8) return JLE_BAD_ARG;
+  dim3 g((unsigned)((items + 3) / 4)), b(256);
+#define JLE_LATENT_MFMA(NRV)                                                                                        \
+  hipLaunchKernelGGL(latent_attention_mfma_kernel<NRV>, g, b, 0, s, (const bf16_t*)q_lat, (const bf16_t*)q, q_ld,   \
+                     dn, dr, (const bf16_t*)latent_pages, (const bf16_t*)latent_t_pages, (const bf16_t*)rope_pages, \
+                     (bf16_t*)out, positions, token_segment, block_table, table_width, window, scale, tiles,        \
+                     num_tiles, N, H, R, ps, splits, steps_per_split, ws_ml, ws_o)
+  if (R <= 128)
+    JLE_LATENT_MFMA(4);
+  else if (R <= 256)
+    JLE_LATENT_MFMA(8);
+  else
+    JLE_LATENT_MFMA(16);
+#undef JLE_LATENT_MFMA
+  JLE_LAUNCH_CHECK();
+  if (splits > 1) {
+    dim3 gm((unsigned)(((long long)N * H + 3) / 4));
+    hipLaunchKernelGGL(latent_attention_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * H, R, splits);
+    JLE_LAUNCH_CHECK();
+  }
+  return 0;
+}
 
 JLE_API int jle_latent_prepare(void* rows, int ld, int H, int dn, int dr, int R, const int* positions,
                                const float* inv_freq, int pairing, int rd, const float* norm_w, float eps,
-                               void* latent_pages, void* rope_pages, const int* slot_mapping, int writes,
-                               int is_bf16, int N, hipStream_t s) {
+                               void* latent_pages, void* rope_pages, void* latent_t_pages, int ps,
+                               const int* slot_mapping, int writes, int is_bf16, int N, hipStream_t s) {
   if (N <= 0) return 0;
   if (H <= 0 || dn < 0 || dr <= 0 || R <= 0 || rd % 2 || rd < 0 || rd > dr || (rd > 0 && inv_freq == nullptr))
     return JLE_BAD_ARG;
   if (ld < H * (dn + dr) + (writes ? R + dr : 0)) return JLE_BAD_ARG;
-  if (writes && (latent_pages == nullptr || rope_pages == nullptr || slot_mapping == nullptr)) return JLE_BAD_ARG;
+  if (writes && (latent_pages == nullptr || rope_pages == nullptr || slot_mapping == nullptr || ps <= 0))
+    return JLE_BAD_ARG;
   if (is_bf16)
     hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, dim3(N), dim3(256), 0, s, (bf16_t*)rows, ld, H, dn, dr, R,
                        positions, inv_freq, pairing, rd, norm_w, eps, (bf16_t*)latent_pages, (bf16_t*)rope_pages,
-                       slot_mapping, writes);
+                       (bf16_t*)latent_t_pages, ps, slot_mapping, writes);
   else
     hipLaunchKernelGGL(latent_prepare_kernel<float>, dim3(N), dim3(256), 0, s, (float*)rows, ld, H, dn, dr, R,
                        positions, inv_freq, pairing, rd, norm_w, eps, (float*)latent_pages, (float*)rope_pages,
-                       slot_mapping, writes);
+                       (float*)latent_t_pages, ps, slot_mapping, writes);
   JLE_LAUNCH_CHECK();
   return 0;
 }

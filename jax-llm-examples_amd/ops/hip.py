@@ -60,7 +60,9 @@ _SIGNATURES = {
     "jle_add_norm_shift": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                            _vp, _i, _i, _i, _i, _vp],
     "jle_polynorm": [_vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
-    "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
+    "jle_latent_attention_mfma": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
+                                  _i, _i, _i, _i, _vp, _vp, _vp],
     "jle_latent_attention": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i,
                              _vp, _vp, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -127,6 +129,7 @@ def load_library():
             fn.restype = ctypes.c_int
         lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
         lib.jle_gemm_stream_supported.argtypes = [_i, _i, _i]
+        lib.jle_latent_attention_mfma_supported.argtypes = [_i, _i, _i, _i, _i]
         lib.jle_gemm_f32_stream_supported.argtypes = [_i, _i, _i]
         lib.jle_attention_group_waves.argtypes = []
         lib._jle_path = path
@@ -265,7 +268,10 @@ class HipOps:
         return out.transpose(0, 1).contiguous() if tokens_first else out
 
     def latent_prepare(self, rows, num_heads: int, nope_dim: int, rope_dim: int, kv_rank: int, positions, rotation,
-                       latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool) -> None:
+                       latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool,
+                       latent_t_pages=None) -> None:
+        """``latent_t_pages``: a second copy of the latent, per page ``[kv_rank, page_size]`` (the page's tokens
+        side by side), which the matrix-core attention kernel reads for its second product."""
         n, ld = rows.shape
         self._chk(rows, None, None, "projected rows")
         self._chk(positions, torch.int32, (n,), "positions")
@@ -278,20 +284,26 @@ class HipOps:
             np_, ps = latent_pages.shape[0], latent_pages.shape[1]
             self._chk(latent_pages, rows.dtype, (np_, ps, kv_rank), "latent pages")
             self._chk(rope_pages, rows.dtype, (np_, ps, rope_dim), "rotated key pages")
+            if latent_t_pages is not None:
+                self._chk(latent_t_pages, rows.dtype, (np_, ps, kv_rank), "transposed latent pages")
             self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
             if latent_norm is not None:
                 self._chk(latent_norm, torch.float32, (kv_rank,), "latent norm weight")
         self._call("jle_latent_prepare", _p(rows), ld, num_heads, nope_dim, rope_dim, kv_rank, _p(positions), _p(inv),
                    pairing, rd, _p(latent_norm) if writes else None, float(eps),
                    _p(latent_pages) if writes else None, _p(rope_pages) if writes else None,
+                   _p(latent_t_pages) if writes else None, latent_pages.shape[1] if writes else 0,
                    _p(slot_mapping) if writes else None, int(bool(writes)), self._is_bf16(rows), n)
 
     LATENT_SPLIT_BELOW = 2048  # fewer (token, head) pairs than this: a query's key tiles are shared between wavefronts
 
+    LATENT_MFMA_ITEMS = 1024  # the matrix-core kernel: fewer row tiles than this share their key steps between wavefronts
+
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
-                         token_segment, window, scale: float, meta=None):
+                         token_segment, window, scale: float, meta=None, latent_t_pages=None):
         """See ``attention_latent.hip``.  ``q_lat [H, N, kv_rank]``, ``q [N, H, nope + rope]`` (a view of the
-        projected rows: the heads' queries lie at their start); returns ``[N, H, kv_rank]``."""
+        projected rows: the heads' queries lie at their start); returns ``[N, H, kv_rank]``.  In bfloat16, with the
+        latent's transposed copy and sizes that fit, on the matrix cores; else in float32 arithmetic."""
         H, n, r = q_lat.shape
         dr = q.shape[2] - nope_dim
         np_, ps = latent_pages.shape[0], latent_pages.shape[1]
@@ -306,6 +318,11 @@ class HipOps:
         self._chk(token_segment, torch.int32, (n,), "token segments")
         w = 0 if window is None else int(window)
         out = torch.empty(n, H, r, dtype=q_lat.dtype, device=q_lat.device)
+        if (latent_t_pages is not None and q_lat.dtype == torch.bfloat16
+                and self.lib.jle_latent_attention_mfma_supported(r, nope_dim, dr, q_ld, ps)):
+            self._chk(latent_t_pages, latent_pages.dtype, (np_, ps, r), "transposed latent pages")
+            return self._latent_attention_mfma(q_lat, q, q_ld, nope_dim, dr, latent_pages, latent_t_pages, rope_pages,
+                                               out, block_table, positions, token_segment, w, scale, meta)
         splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
         waves = n * H
         if waves < self.LATENT_SPLIT_BELOW:
@@ -326,6 +343,48 @@ class HipOps:
         self._call("jle_latent_attention", _p(q_lat), _p(q), q_ld, nope_dim, dr, _p(latent_pages), _p(rope_pages), _p(out),
                    _p(positions), _p(token_segment), _p(block_table), block_table.shape[1], w, float(scale),
                    self._is_bf16(q_lat), n, H, r, ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
+        return out
+
+    def _latent_attention_mfma(self, q_lat, q, q_ld, dn, dr, latent_pages, latent_t_pages, rope_pages, out,
+                               block_table, positions, token_segment, window, scale, meta):
+        H, n, r = q_lat.shape
+        ps = latent_pages.shape[1]
+        # row tiles: 16 consecutive (token, head) pairs of one segment
+        key = f"latent_tiles_{H}"
+        plan = meta.meta.get(key) if meta is not None else None
+        if plan is None:
+            seg_lens = meta.seg_lens if meta is not None and meta.seg_lens else \
+                self._segments(meta, token_segment, positions)[0]
+            flat, o = [], 0
+            for ln in seg_lens:
+                rows = ln * H
+                for t in range(0, rows, 16):
+                    flat += [o * H + t, min(16, rows - t)]
+                o += ln
+            plan = torch.tensor(flat, dtype=torch.int32).to(q_lat.device)
+            if meta is not None:
+                meta.meta[key] = plan
+        tiles = plan.numel() // 2
+        splits, steps_per_split, ws_ml, ws_o = 1, 0, None, None
+        if tiles < self.LATENT_MFMA_ITEMS:
+            if meta is not None and meta.decode_bucket is not None:
+                longest = meta.decode_bucket  # (a step of single tokens: laid out for the bound, see GroupContext)
+            elif meta is not None and meta.seg_starts is not None:
+                longest = max(s0 + ln for s0, ln in zip(meta.seg_starts, meta.seg_lens))
+            else:
+                longest = int(positions.max()) + 1
+            span = min(window, longest) if window else longest
+            spanned = -(-16 // H) + 1 if H < 16 else 1  # tokens whose rows may share a tile
+            steps = -(-(span + spanned + 31) // 32)
+            want = min(steps, -(-self.LATENT_MFMA_ITEMS // tiles))
+            if want > 1:
+                steps_per_split = -(-steps // want)
+                splits = -(-steps // steps_per_split)
+                ws_ml = torch.empty(n * H * splits * 2, dtype=torch.float32, device=q_lat.device)
+                ws_o = torch.empty(n * H * splits * r, dtype=torch.float32, device=q_lat.device)
+        self._call("jle_latent_attention_mfma", _p(q_lat), _p(q), q_ld, dn, dr, _p(latent_pages), _p(latent_t_pages),
+                   _p(rope_pages), _p(out), _p(positions), _p(token_segment), _p(block_table), block_table.shape[1],
+                   window, float(scale), _p(plan), tiles, n, H, r, ps, splits, steps_per_split, _p(ws_ml), _p(ws_o))
         return out
 
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):

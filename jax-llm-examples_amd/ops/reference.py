@@ -147,7 +147,8 @@ class ReferenceOps:
         return torch.cat([head, rest], dim=-1)
 
     def latent_prepare(self, rows, num_heads: int, nope_dim: int, rope_dim: int, kv_rank: int, positions, rotation,
-                       latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool) -> None:
+                       latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool,
+                       latent_t_pages=None) -> None:
         """``rows``: ``[N, H * (nope + rope) (+ kv_rank + rope)]``.  Turns the ``rope`` part of every head's
         query in place; if the run writes its cache: RMS-norms the latent (the ``kv_rank`` numbers behind the
         queries) with ``latent_norm``, turns the shared key part (the last ``rope`` numbers) and writes both
@@ -166,9 +167,11 @@ class ReferenceOps:
             page, off = (slot_mapping // ps).long(), (slot_mapping % ps).long()
             latent_pages[page, off] = c.to(latent_pages.dtype)
             rope_pages[page, off] = kr.to(rope_pages.dtype)
+            if latent_t_pages is not None:  # a second copy, per page [kv_rank, page_size]
+                latent_t_pages.view(latent_t_pages.shape[0], kv_rank, ps)[page, :, off] = c.to(latent_t_pages.dtype)
 
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
-                         token_segment, window, scale: float, meta=None):
+                         token_segment, window, scale: float, meta=None, latent_t_pages=None):
         """For every token and head: softmax over the visible cached tokens ``j`` (``0 <= pos - j < window``;
         all earlier ones without a window) of ``(q_lat . c_j + q_r . k_j) * scale``, and the sum of the ``c_j``
         with those weights.  ``q_lat``: ``[H, N, kv_rank]``; ``q``: ``[N, H, nope + rope]`` whose rotated part is

@@ -63,8 +63,21 @@ class LatentAttention(Mixer):
             specs["latent_norm"] = ParamSpec((self.kv_rank,), policy="float32", init=("uniform", 0.5, 1.5))
         return specs
 
+    def allocate(self, dtype, device) -> None:
+        super().allocate(dtype, device)
+        # In bfloat16, at sizes the matrix-core attention kernel takes, the cache holds the latent twice: token by
+        # token for the scores, and per page with the page's tokens side by side for the weighted sum.
+        self.transposed_copy = (dtype == torch.bfloat16 and self.kv_rank % 32 == 0 and self.kv_rank <= 512
+                                and self.rope_dim % 8 == 0 and self.rope_dim <= 64)  # (of the cache's sizes alone:
+        # every run that shares the cache must say the same)
+
+    transposed_copy = False
+
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(paged=(("latent", (self.kv_rank,)), ("rope_key", (self.rope_dim,))), retention=self.retention)
+        paged = (("latent", (self.kv_rank,)), ("rope_key", (self.rope_dim,)))
+        if self.transposed_copy:
+            paged += (("latent_t", (self.kv_rank,)),)
+        return CacheNeed(paged=paged, retention=self.retention)
 
     graph_safe = True
 
@@ -95,13 +108,14 @@ class LatentAttention(Mixer):
         # rotates q_r in place, norms the latent, rotates the shared key part and writes both into their pages
         ops.latent_prepare(rows, H, dn, dr, r, ctx.positions, self.rotation,
                            self.params.get("latent_norm"), self.latent_norm_eps,
-                           cache.pages["latent"], cache.pages["rope_key"], cache.slot_mapping, cache.writes)
+                           cache.pages["latent"], cache.pages["rope_key"], cache.slot_mapping, cache.writes,
+                           latent_t_pages=cache.pages.get("latent_t"))
         q = rows[:, : self.q_rows].view(n, H, dn + dr)
         # queries into the latent's space: [H, N, dn] x [H, dn, r]
         q_lat = ops.batched_linear(q[:, :, :dn].transpose(0, 1), self.params["w_uk"].view(H, dn, r))
         o_lat = ops.latent_attention(q_lat, q, dn, cache.pages["latent"], cache.pages["rope_key"], cache.block_table,
                                      ctx.positions, ctx.token_segment, self.window, self.softmax_scale,
-                                     cache.attn_meta)  # [N, H, r]
+                                     cache.attn_meta, latent_t_pages=cache.pages.get("latent_t"))  # [N, H, r]
         # the sums out of it: [H, N, r] x [H, r, dv], laid out [N, H * dv]
         o = ops.batched_linear(o_lat.transpose(0, 1), self.params["w_uv"].view(H, dv, r).transpose(1, 2), tokens_first=True)
         return ops.linear(o.view(n, H * dv), self.params["wo"])
