@@ -416,7 +416,244 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   }
 }
 
+
+// The same computation for steps of many tokens: the four wavefronts of a block take four neighbouring row tiles
+// (64 consecutive (token, head) rows of one segment), whose keys are nearly the same, and share every step's 32
+// keys through shared memory: the block brings the keys' rows ([32][kv_rank + rope], rope padded with zeros to a
+// multiple of 32) and the transposed latent ([kv_rank][32]) in once, each wavefront reads its operands from there.
+// The next step's data is asked for into registers before this step's products start and stored after them.
+template <int NR>
+__global__ __launch_bounds__(256) void latent_attention_lds_kernel(
+    const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ q, int q_ld, int dn, int dr,
+    const bf16_t* __restrict__ latent, const bf16_t* __restrict__ latent_t, const bf16_t* __restrict__ rope,
+    bf16_t* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_segment,
+    const int* __restrict__ block_table, int table_width, int window, float scale, const int* __restrict__ blocks,
+    int N, int H, int R, int ps) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int drp = (dr + 31) & ~31;
+  const int KS = R + drp + 8, VS = 40;  // row pitches in elements (16 bytes of padding: no bank conflicts)
+  bf16_t* sk = reinterpret_cast<bf16_t*>(smem_raw);  // [32][KS]
+  bf16_t* sv = sk + 32 * KS;                         // [R][VS]
+  const int tid = threadIdx.x, lane = tid & 63, g = lane >> 4, r = lane & 15;
+  const int w = wave_index();
+  const int brow0 = blocks[2 * blockIdx.x], bnrows = blocks[2 * blockIdx.x + 1];
+  const int n_first = brow0 / H, n_last = (brow0 + bnrows - 1) / H;
+  const int bhi = positions[n_last];
+  const int pos_first = positions[n_first];
+  const int blo = window > 0 ? max(0, pos_first - window + 1) : 0;
+  const int* table = block_table + (size_t)token_segment[n_first] * table_width;
+  // this wavefront's tile
+  const int nrows = min(16, bnrows - 16 * w);
+  const bool active = nrows > 0;
+  const bool row_ok = r < nrows;
+  const int row = brow0 + (row_ok ? 16 * w + r : 0);
+  const int n = row / H, h = row - n * H;
+  const int pos = positions[n];
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  int lo = row_ok ? first : 0x7fffffff, hi = row_ok ? pos : -1;
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) {
+    lo = min(lo, __shfl_xor(lo, o, 64));
+    hi = max(hi, __shfl_xor(hi, o, 64));
+  }
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  bf16x8 qb[NR + 2];
+  {
+    const bf16_t* ql = q_lat + ((size_t)h * N + n) * R;
+#pragma unroll
+    for (int c = 0; c < NR; ++c) {
+      const int k0 = c * 32 + g * 8;
+      qb[c] = __builtin_bit_cast(bf16x8, k0 < R ? load16(ql + k0) : zero4);
+    }
+    const bf16_t* qr = q + (size_t)n * q_ld + (size_t)h * (dn + dr) + dn;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int k0 = c * 32 + g * 8;
+      qb[NR + c] = __builtin_bit_cast(bf16x8, k0 < dr ? load16(qr + k0) : zero4);
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[NR * 2];
+#pragma unroll
+  for (int dt = 0; dt < NR * 2; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // what this thread brings in per step: pieces of 16 bytes
+  constexpr int KMAX = (NR * 4 + 8 + 7) / 8;  // 32 keys x (R + drp) / 8 pieces over 256 threads
+  constexpr int VMAX = (NR + 1) / 2;          // R x 4 pieces over 256 threads
+  const int KC = (R + drp) >> 3;              // pieces per key
+  int k_key[KMAX], k_col[KMAX];
+#pragma unroll
+  for (int i = 0; i < KMAX; ++i) {
+    const int id = tid + 256 * i;
+    k_key[i] = id / KC;
+    k_col[i] = (id - k_key[i] * KC) * 8;
+  }
+  u32x4 stage_k[KMAX], stage_v[VMAX];
+  auto prefetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i) {
+      u32x4 v = zero4;
+      if (k_key[i] < 32) {
+        const int key = t0 + k_key[i];
+        const int page = key <= bhi ? table[key / ps] : -1;
+        if (page >= 0) {
+          const size_t slot = (size_t)page * ps + key % ps;
+          const int col = k_col[i];
+          if (col < R) v = load16(latent + slot * R + col);
+          else if (col - R < dr) v = load16(rope + slot * dr + (col - R));
+        }
+      }
+      stage_k[i] = v;
+    }
+#pragma unroll
+    for (int j = 0; j < VMAX; ++j) {
+      const int id = tid + 256 * j;
+      const int d = id >> 2, kq = id & 3;
+      u32x4 v = zero4;
+      if (d < R) {
+        const int key0 = t0 + 8 * kq;
+        const int page = key0 <= bhi ? table[key0 / ps] : -1;
+        if (page >= 0) {
+          v = load16(latent_t + ((size_t)page * R + d) * ps + key0 % ps);
+          const int n_ok = min(8, bhi - key0 + 1);  // (tokens behind the block's last position are not written yet)
+#pragma unroll
+          for (int w2 = 0; w2 < 4; ++w2)
+            v[w2] &= n_ok >= 2 * w2 + 2 ? 0xffffffffu : (n_ok == 2 * w2 + 1 ? 0x0000ffffu : 0u);
+        }
+      }
+      stage_v[j] = v;
+    }
+  };
+  const int t_first = (blo / 32) * 32;
+  prefetch(t_first);
+  for (int t0 = t_first; t0 <= bhi; t0 += 32) {
+    __syncthreads();  // everyone has read the step before
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i)
+      if (k_key[i] < 32) *reinterpret_cast<u32x4*>(sk + k_key[i] * KS + k_col[i]) = stage_k[i];
+#pragma unroll
+    for (int j = 0; j < VMAX; ++j) {
+      const int id = tid + 256 * j;
+      if ((id >> 2) < R) *reinterpret_cast<u32x4*>(sv + (id >> 2) * VS + (id & 3) * 8) = stage_v[j];
+    }
+    __syncthreads();
+    if (t0 + 32 <= bhi) prefetch(t0 + 32);
+    if (!active || t0 + 31 < lo || t0 > hi) continue;  // none of this tile's rows sees a key of the step
+    f32x4 st[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* arow = sk + (8 * (r >> 2) + 4 * t + (r & 3)) * KS + g * 8;
+#pragma unroll
+      for (int c = 0; c < NR; ++c)
+        if (c * 32 < R)
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, load16(arow + c * 32)), qb[c],
+                                                          st[t], 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        if (c * 32 < dr)
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, load16(arow + R + c * 32)),
+                                                          qb[NR + c], st[t], 0, 0, 0);
+    }
+    float sv8[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = t0 + 8 * g + e;
+      const bool ok = row_ok && key >= first && key <= pos;
+      sv8[e] = ok ? st[e >> 2][e & 3] * scale : -INFINITY;
+      mx = fmaxf(mx, sv8[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float p[8];
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = sv8[e] == -INFINITY ? 0.f : expf(sv8[e] - m_new);
+      psum += p[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+    const u32x4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+    const bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
+    const bf16_t* vrow = sv + r * VS + g * 8;
+#pragma unroll
+    for (int dt = 0; dt < NR * 2; ++dt) {
+      if (dt * 16 < R) {
+        acc[dt] *= corr;
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, load16(vrow + dt * 16 * VS)), pb,
+                                                          acc[dt], 0, 0, 0);
+      }
+    }
+  }
+  if (!row_ok) return;
+  const float inv = 1.0f / l;
+  bf16_t* o = out + (size_t)row * R;
+#pragma unroll
+  for (int dt = 0; dt < NR * 2; ++dt) {
+    if (dt * 16 < R) {
+      const uint2 w2 = {pack_bf16(acc[dt][0] * inv, acc[dt][1] * inv), pack_bf16(acc[dt][2] * inv, acc[dt][3] * inv)};
+      *reinterpret_cast<uint2*>(o + dt * 16 + g * 4) = w2;
+    }
+  }
+}
+
+template <int NR>
+int launch_latent_lds(dim3 grid, size_t smem, hipStream_t s, const bf16_t* q_lat, const bf16_t* q, int q_ld, int dn,
+                      int dr, const bf16_t* latent, const bf16_t* latent_t, const bf16_t* rope, bf16_t* out,
+                      const int* positions, const int* token_segment, const int* block_table, int table_width,
+                      int window, float scale, const int* blocks, int N, int H, int R, int ps) {
+  static size_t allowed = 0;  // (what this kernel has been given leave to use of the compute unit's shared memory)
+  if (smem > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_lds_kernel<NR>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return (int)e;
+    allowed = smem;
+  }
+  hipLaunchKernelGGL(latent_attention_lds_kernel<NR>, grid, dim3(256), smem, s, q_lat, q, q_ld, dn, dr, latent,
+                     latent_t, rope, out, positions, token_segment, block_table, table_width, window, scale, blocks, N,
+                     H, R, ps);
+  return 0;
+}
+
 }  // namespace
+
+// blocks: (first row, rows) pairs, up to 64 consecutive rows (token * H + head) of one segment each.
+JLE_API int jle_latent_attention_lds(const void* q_lat, const void* q, int q_ld, int dn, int dr,
+                                     const void* latent_pages, const void* latent_t_pages, const void* rope_pages,
+                                     void* out, const int* positions, const int* token_segment,
+                                     const int* block_table, int table_width, int window, float scale,
+                                     const int* blocks, int num_blocks, int N, int H, int R, int ps, hipStream_t s) {
+  if (N <= 0 || num_blocks <= 0) return 0;
+  if (!(R > 0 && R % 32 == 0 && R <= 512 && dr > 0 && dr % 8 == 0 && dr <= 64 && dn % 8 == 0 && q_ld % 8 == 0 &&
+        ps % 8 == 0) ||
+      H <= 0 || window < 0 || blocks == nullptr || latent_t_pages == nullptr || q_ld < H * (dn + dr))
+    return JLE_BAD_ARG;
+  const int drp = (dr + 31) & ~31;
+  const size_t smem = (size_t)(32 * (R + drp + 8) + R * 40) * sizeof(bf16_t);
+  dim3 grid((unsigned)num_blocks);
+  int rc;
+#define JLE_LATENT_LDS(NRV)                                                                                        \
+  rc = launch_latent_lds<NRV>(grid, smem, s, (const bf16_t*)q_lat, (const bf16_t*)q, q_ld, dn, dr,                 \
+                              (const bf16_t*)latent_pages, (const bf16_t*)latent_t_pages, (const bf16_t*)rope_pages, \
+                              (bf16_t*)out, positions, token_segment, block_table, table_width, window, scale, blocks, \
+                              N, H, R, ps)
+  if (R <= 128)
+    JLE_LATENT_LDS(4);
+  else if (R <= 256)
+    JLE_LATENT_LDS(8);
+  else
+    JLE_LATENT_LDS(16);
+#undef JLE_LATENT_LDS
+  if (rc != 0) return rc;
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
 
 // Whether the matrix-core kernel takes these sizes (bfloat16 only): rows read 16 bytes at a time.
 JLE_API int jle_latent_attention_mfma_supported(int R, int dn, int dr, int q_ld, int ps) {

@@ -61,6 +61,8 @@ _SIGNATURES = {
                            _vp, _i, _i, _i, _i, _vp],
     "jle_polynorm": [_vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
     "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
+    "jle_latent_attention_lds": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
+                                 _i, _i, _vp],
     "jle_latent_attention_mfma": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
                                   _i, _i, _i, _i, _vp, _vp, _vp],
     "jle_latent_attention": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i,
@@ -298,6 +300,7 @@ class HipOps:
     LATENT_SPLIT_BELOW = 2048  # fewer (token, head) pairs than this: a query's key tiles are shared between wavefronts
 
     LATENT_MFMA_ITEMS = 1024  # the matrix-core kernel: fewer row tiles than this share their key steps between wavefronts
+    LATENT_LDS_TILES = 1024  # from so many row tiles on: the kernel whose blocks share keys through shared memory
 
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
                          token_segment, window, scale: float, meta=None, latent_t_pages=None):
@@ -365,6 +368,26 @@ class HipOps:
             if meta is not None:
                 meta.meta[key] = plan
         tiles = plan.numel() // 2
+        if tiles >= self.LATENT_LDS_TILES:
+            # many rows: blocks of four neighbouring tiles that share their keys through shared memory
+            key = f"latent_blocks_{H}"
+            blocks = meta.meta.get(key) if meta is not None else None
+            if blocks is None:
+                seg_lens = meta.seg_lens if meta is not None and meta.seg_lens else \
+                    self._segments(meta, token_segment, positions)[0]
+                flat, o = [], 0
+                for ln in seg_lens:
+                    rows = ln * H
+                    for t in range(0, rows, 64):
+                        flat += [o * H + t, min(64, rows - t)]
+                    o += ln
+                blocks = torch.tensor(flat, dtype=torch.int32).to(q_lat.device)
+                if meta is not None:
+                    meta.meta[key] = blocks
+            self._call("jle_latent_attention_lds", _p(q_lat), _p(q), q_ld, dn, dr, _p(latent_pages),
+                       _p(latent_t_pages), _p(rope_pages), _p(out), _p(positions), _p(token_segment), _p(block_table),
+                       block_table.shape[1], window, float(scale), _p(blocks), blocks.numel() // 2, n, H, r, ps)
+            return out
         splits, steps_per_split, ws_ml, ws_o = 1, 0, None, None
         if tiles < self.LATENT_MFMA_ITEMS:
             if meta is not None and meta.decode_bucket is not None:

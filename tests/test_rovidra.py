@@ -296,6 +296,19 @@ def test_gpu_bfloat16(folders_bf16, name, mode):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["RA", "RF"])
+def test_gpu_bfloat16_with_keys_shared_through_shared_memory(folders_bf16, monkeypatch, name, mode):
+    """Steps of many tokens go through the attention kernel whose blocks share their keys; here every step of more
+    than a few rows does (tiles of several tokens, blocks that end inside a segment, windows that start inside a
+    step of 32 keys)."""
+    from jax_llm_examples_amd.ops.hip import HipOps
+
+    monkeypatch.setattr(HipOps, "LATENT_LDS_TILES", 2)
+    _check(name, folders_bf16[name], "bfloat16", "cuda:0", mode)
+
+
+@pytest.mark.gpu
 def test_gpu_float32_at_vector_sizes(tmp_path):
     folder = write_rovidra("RF", str(tmp_path / "RF"), torch.float32)
     for mode in ("portions", "mixed"):
