@@ -230,16 +230,30 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float
   float acc[kMaxAcc];
 #pragma unroll
   for (int i = 0; i < kMaxAcc; ++i) acc[i] = 0.f;
-  for (int sp = 0; sp < splits; ++sp) {
-    const float ms = ml[sp * 2], ls = ml[sp * 2 + 1];
-    if (ms == -INFINITY || ms != ms) continue;  // a range without keys
-    const float wgt = expf(ms - mx);
-    l += ls * wgt;
-    const float* row = ws_o + ((size_t)nh * splits + sp) * R;
+  // the sums in the ranges' order; four ranges' rows are asked for before the first is added
+  constexpr int U = 4;
+  for (int s0 = 0; s0 < splits; s0 += U) {
+    float ms[U], ls[U], o[U][kMaxAcc];
 #pragma unroll
-    for (int i = 0; i < kMaxAcc; ++i) {
-      const int d = lane + 64 * i;
-      if (d < R) acc[i] = __builtin_fmaf(row[d], wgt, acc[i]);
+    for (int u = 0; u < U; ++u) {
+      const int sp = min(s0 + u, splits - 1);  // (past the last: loaded again, not used)
+      ms[u] = ml[sp * 2];
+      ls[u] = ml[sp * 2 + 1];
+      const float* row = ws_o + ((size_t)nh * splits + sp) * R;
+#pragma unroll
+      for (int i = 0; i < kMaxAcc; ++i) {
+        const int d = lane + 64 * i;
+        o[u][i] = d < R ? row[d] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (s0 + u >= splits) break;
+      if (ms[u] == -INFINITY || ms[u] != ms[u]) continue;  // a range without keys
+      const float wgt = expf(ms[u] - mx);
+      l += ls[u] * wgt;
+#pragma unroll
+      for (int i = 0; i < kMaxAcc; ++i) acc[i] = __builtin_fmaf(o[u][i], wgt, acc[i]);
     }
   }
   const float inv = bad ? __builtin_nanf("") : 1.0f / l;
@@ -323,28 +337,32 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const int key = t0 + 8 * (r >> 2) + 4 * t + (r & 3);  // which key is row r of this A operand
-      const int page = key <= hi ? table[key / ps] : -1;
-      const bool have = page >= 0;
-      const size_t slot = have ? (size_t)page * ps + key % ps : 0;
+      // which key is row r of this A operand; every load is made (from a place that exists) and what must not
+      // count is put to zero afterwards: a load under a branch would wait for the one before it
+      const int key = t0 + 8 * (r >> 2) + 4 * t + (r & 3);
+      const int page = table[min(key, hi) / ps];
+      const bool have = key <= hi && page >= 0;
+      const size_t slot = (size_t)max(page, 0) * ps + key % ps;
       const bf16_t* crow = latent + slot * R;
       const bf16_t* krow = rope + slot * dr;
+      // (no branch in these loops, not even one that all lanes take alike: loads on the far side of a branch are
+      // not asked for before the products on this side are done; a chunk past the latent's width is a product
+      // with zeros)
+      u32x4 ka[NR + 2];
 #pragma unroll
       for (int c = 0; c < NR; ++c) {
-        if (c * 32 < R) {
-          const int k0 = c * 32 + g * 8;
-          const bf16x8 a = __builtin_bit_cast(bf16x8, (have && k0 < R) ? load16(crow + k0) : zero4);
-          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[c], st[t], 0, 0, 0);
-        }
+        ka[c] = load16(crow + min(c * 32, R - 32) + g * 8);
+        if (!have || c * 32 >= R) ka[c] = zero4;
       }
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        if (c * 32 < dr) {
-          const int k0 = c * 32 + g * 8;
-          const bf16x8 a = __builtin_bit_cast(bf16x8, (have && k0 < dr) ? load16(krow + k0) : zero4);
-          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[NR + c], st[t], 0, 0, 0);
-        }
+        const int k0 = c * 32 + g * 8;
+        ka[NR + c] = load16(krow + min(k0, dr - 8));
+        if (!have || k0 >= dr) ka[NR + c] = zero4;
       }
+#pragma unroll
+      for (int c = 0; c < NR + 2; ++c)
+        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[c]), qb[c], st[t], 0, 0, 0);
     }
     // this lane now holds, for its row, the scores of keys t0 + 8 g .. + 7
     float sv[8];
@@ -376,21 +394,24 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     // the latent's transposed copy: row d of a page holds its tokens side by side
     const int key0 = t0 + 8 * g;
     const int vpage = key0 <= hi ? table[key0 / ps] : -1;
-    const bf16_t* vbase = latent_t + ((size_t)(vpage < 0 ? 0 : vpage) * R + r) * ps + key0 % ps;
+    const bf16_t* vbase = latent_t + ((size_t)max(vpage, 0) * R + r) * ps + key0 % ps;
     // tokens behind the rows' last position are not written yet: what lies there must not meet a zero weight
     const int n_ok = min(8, hi - key0 + 1);
+    const bool rescale = !__all(corr == 1.f);  // (only when some row's maximum moved)
     u32x4 keep;
 #pragma unroll
     for (int w2 = 0; w2 < 4; ++w2)
-      keep[w2] = n_ok >= 2 * w2 + 2 ? 0xffffffffu : (n_ok == 2 * w2 + 1 ? 0x0000ffffu : 0u);
+      keep[w2] = vpage < 0 ? 0u : (n_ok >= 2 * w2 + 2 ? 0xffffffffu : (n_ok == 2 * w2 + 1 ? 0x0000ffffu : 0u));
+    if (rescale) {
+#pragma unroll
+      for (int dt = 0; dt < NR * 2; ++dt) acc[dt] *= corr;
+    }
 #pragma unroll
     for (int dt = 0; dt < NR * 2; ++dt) {
-      if (dt * 16 < R) {
-        u32x4 v = vpage >= 0 ? load16(vbase + (size_t)dt * 16 * ps) : zero4;
-        v &= keep;
-        acc[dt] *= corr;
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, acc[dt], 0, 0, 0);
-      }
+      u32x4 v = load16(vbase + (size_t)min(dt * 16, R - 16) * ps);
+      v &= keep;
+      if (dt * 16 >= R) v = zero4;
+      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, acc[dt], 0, 0, 0);
     }
   }
   if (!row_ok) return;
@@ -432,8 +453,10 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int drp = (dr + 31) & ~31;
   const int KS = R + drp + 8, VS = 40;  // row pitches in elements (16 bytes of padding: no bank conflicts)
-  bf16_t* sk = reinterpret_cast<bf16_t*>(smem_raw);  // [32][KS]
+  const int QS = R + 8;
+  bf16_t* sk = reinterpret_cast<bf16_t*>(smem_raw);  // [32][KS]: key t0 + kk in row key_row(kk)
   bf16_t* sv = sk + 32 * KS;                         // [R][VS]
+  bf16_t* sq = sv + R * VS;                          // [64][QS]: the rows' queries in the latent's space
   const int tid = threadIdx.x, lane = tid & 63, g = lane >> 4, r = lane & 15;
   const int w = wave_index();
   const int brow0 = blocks[2 * blockIdx.x], bnrows = blocks[2 * blockIdx.x + 1];
@@ -457,71 +480,73 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
     hi = max(hi, __shfl_xor(hi, o, 64));
   }
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
-  bf16x8 qb[NR + 2];
+  // the queries: the rotated part stays in registers, the part in the latent's space (up to 16 operands a row)
+  // lies in shared memory and is read again every step - the registers it would take are what the next step's
+  // data waits in
+  bf16x8 qrot[2];
   {
     const bf16_t* ql = q_lat + ((size_t)h * N + n) * R;
+    bf16_t* mine = sq + (16 * w + r) * QS;
 #pragma unroll
     for (int c = 0; c < NR; ++c) {
       const int k0 = c * 32 + g * 8;
-      qb[c] = __builtin_bit_cast(bf16x8, k0 < R ? load16(ql + k0) : zero4);
+      if (k0 < R) *reinterpret_cast<u32x4*>(mine + k0) = load16(ql + k0);
     }
     const bf16_t* qr = q + (size_t)n * q_ld + (size_t)h * (dn + dr) + dn;
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
       const int k0 = c * 32 + g * 8;
-      qb[NR + c] = __builtin_bit_cast(bf16x8, k0 < dr ? load16(qr + k0) : zero4);
+      u32x4 v = load16(qr + min(k0, dr - 8));
+      if (k0 >= dr) v = zero4;
+      qrot[c] = __builtin_bit_cast(bf16x8, v);
     }
   }
+  const bf16_t* qrow = sq + (16 * w + r) * QS + g * 8;
   float m = -INFINITY, l = 0.f;
   f32x4 acc[NR * 2];
 #pragma unroll
   for (int dt = 0; dt < NR * 2; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // what this thread brings in per step: pieces of 16 bytes
-  constexpr int KMAX = (NR * 4 + 8 + 7) / 8;  // 32 keys x (R + drp) / 8 pieces over 256 threads
+  // what this thread brings in per step, in pieces of 16 bytes: of the keys' rows, eight threads take a key and
+  // every eighth piece of its row each; of the transposed latent, four threads take a row of 32 tokens
+  constexpr int KMAX = (NR * 4 + 8 + 7) / 8;  // (R + drp) / 8 pieces per key over 8 threads
   constexpr int VMAX = (NR + 1) / 2;          // R x 4 pieces over 256 threads
   const int KC = (R + drp) >> 3;              // pieces per key
-  int k_key[KMAX], k_col[KMAX];
-#pragma unroll
-  for (int i = 0; i < KMAX; ++i) {
-    const int id = tid + 256 * i;
-    k_key[i] = id / KC;
-    k_col[i] = (id - k_key[i] * KC) * 8;
-  }
+  const int k_key = tid >> 3, k_piece = tid & 7;
+  // key kk of a step lies in row (kk >> 2 & 1) * 16 + (kk >> 3) * 4 + (kk & 3): the 16 rows of an A operand are
+  // neighbours, which with this pitch spreads a read over all banks
+  const int k_row = ((k_key >> 2) & 1) * 16 + (k_key >> 3) * 4 + (k_key & 3);
   u32x4 stage_k[KMAX], stage_v[VMAX];
   auto prefetch = [&](int t0) {
+    // lane j (of every wavefront) looks up the page of key t0 + (j & 31); the pieces' pages come from there.  Every
+    // load is made, from a place that exists, and what must not count is put to zero afterwards: a load under a
+    // branch would wait for the one before it.
+    const int mykey = t0 + (lane & 31);
+    const int mypage = table[min(mykey, bhi) / ps];
+    const int mine = mykey <= bhi ? mypage : -1;
+    const int page = __shfl(mine, k_key, 64);
+    const size_t slot = (size_t)max(page, 0) * ps + (t0 + k_key) % ps;
 #pragma unroll
     for (int i = 0; i < KMAX; ++i) {
-      u32x4 v = zero4;
-      if (k_key[i] < 32) {
-        const int key = t0 + k_key[i];
-        const int page = key <= bhi ? table[key / ps] : -1;
-        if (page >= 0) {
-          const size_t slot = (size_t)page * ps + key % ps;
-          const int col = k_col[i];
-          if (col < R) v = load16(latent + slot * R + col);
-          else if (col - R < dr) v = load16(rope + slot * dr + (col - R));
-        }
-      }
+      const int col = min(k_piece + 8 * i, KC - 1) * 8;
+      const bf16_t* src = col < R ? latent + slot * R + col : rope + slot * dr + min(col - R, dr - 8);
+      u32x4 v = load16(src);
+      if (page < 0 || col - R >= dr) v = zero4;
       stage_k[i] = v;
     }
+    const int kq = tid & 3;  // (the same for all of this thread's pieces of the transposed latent)
+    const int key0 = t0 + 8 * kq;
+    const int vpage = __shfl(mine, 8 * kq, 64);
+    const int n_ok = min(8, bhi - key0 + 1);  // (tokens behind the block's last position are not written yet)
+    u32x4 keep;
+#pragma unroll
+    for (int w2 = 0; w2 < 4; ++w2)
+      keep[w2] = vpage < 0 ? 0u : (n_ok >= 2 * w2 + 2 ? 0xffffffffu : (n_ok == 2 * w2 + 1 ? 0x0000ffffu : 0u));
+    const bf16_t* vsrc = latent_t + (size_t)max(vpage, 0) * R * ps + key0 % ps;
 #pragma unroll
     for (int j = 0; j < VMAX; ++j) {
-      const int id = tid + 256 * j;
-      const int d = id >> 2, kq = id & 3;
-      u32x4 v = zero4;
-      if (d < R) {
-        const int key0 = t0 + 8 * kq;
-        const int page = key0 <= bhi ? table[key0 / ps] : -1;
-        if (page >= 0) {
-          v = load16(latent_t + ((size_t)page * R + d) * ps + key0 % ps);
-          const int n_ok = min(8, bhi - key0 + 1);  // (tokens behind the block's last position are not written yet)
-#pragma unroll
-          for (int w2 = 0; w2 < 4; ++w2)
-            v[w2] &= n_ok >= 2 * w2 + 2 ? 0xffffffffu : (n_ok == 2 * w2 + 1 ? 0x0000ffffu : 0u);
-        }
-      }
-      stage_v[j] = v;
+      const int d = min((tid + 256 * j) >> 2, R - 1);
+      stage_v[j] = load16(vsrc + (size_t)d * ps) & keep;
     }
   };
   const int t_first = (blo / 32) * 32;
@@ -530,7 +555,7 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
     __syncthreads();  // everyone has read the step before
 #pragma unroll
     for (int i = 0; i < KMAX; ++i)
-      if (k_key[i] < 32) *reinterpret_cast<u32x4*>(sk + k_key[i] * KS + k_col[i]) = stage_k[i];
+      if (k_piece + 8 * i < KC) *reinterpret_cast<u32x4*>(sk + k_row * KS + (k_piece + 8 * i) * 8) = stage_k[i];
 #pragma unroll
     for (int j = 0; j < VMAX; ++j) {
       const int id = tid + 256 * j;
@@ -543,17 +568,31 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* arow = sk + (8 * (r >> 2) + 4 * t + (r & 3)) * KS + g * 8;
+      const bf16_t* arow = sk + (16 * t + r) * KS + g * 8;
+      // (no branch in these loops: reads on the far side of a branch are not asked for before the products on this
+      // side are done; a chunk past the latent's width is a product with zeros)
 #pragma unroll
-      for (int c = 0; c < NR; ++c)
-        if (c * 32 < R)
-          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, load16(arow + c * 32)), qb[c],
-                                                          st[t], 0, 0, 0);
+      for (int c0 = 0; c0 < NR; c0 += 2) {  // two chunks' reads under way at a time, no more: registers
+        u32x4 a[2], b[2];
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-        if (c * 32 < dr)
-          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, load16(arow + R + c * 32)),
-                                                          qb[NR + c], st[t], 0, 0, 0);
+        for (int u = 0; u < 2; ++u) {
+          const int c = c0 + u;
+          a[u] = load16(arow + min(c * 32, R - 32));
+          b[u] = load16(qrow + min(c * 32, R - 32));
+          if (c * 32 >= R) a[u] = zero4;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]),
+                                                          __builtin_bit_cast(bf16x8, b[u]), st[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        u32x4 a = load16(arow + R + min(c * 32, drp - 32));
+        if (c * 32 >= drp) a = zero4;
+        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qrot[c], st[t], 0, 0, 0);
+      }
     }
     float sv8[8];
     float mx = -INFINITY;
@@ -582,13 +621,22 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
     const u32x4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
     const bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
     const bf16_t* vrow = sv + r * VS + g * 8;
+    if (!__all(corr == 1.f)) {  // (only when some row's maximum moved)
 #pragma unroll
-    for (int dt = 0; dt < NR * 2; ++dt) {
-      if (dt * 16 < R) {
-        acc[dt] *= corr;
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, load16(vrow + dt * 16 * VS)), pb,
-                                                          acc[dt], 0, 0, 0);
+      for (int dt = 0; dt < NR * 2; ++dt) acc[dt] *= corr;
+    }
+#pragma unroll
+    for (int d0 = 0; d0 < NR * 2; d0 += 4) {  // four operands under way at a time
+      u32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        v[u] = load16(vrow + min((d0 + u) * 16, R - 16) * VS);
+        if ((d0 + u) * 16 >= R) v[u] = zero4;
       }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        acc[d0 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v[u]), pb, acc[d0 + u], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   if (!row_ok) return;
@@ -635,7 +683,7 @@ JLE_API int jle_latent_attention_lds(const void* q_lat, const void* q, int q_ld,
       H <= 0 || window < 0 || blocks == nullptr || latent_t_pages == nullptr || q_ld < H * (dn + dr))
     return JLE_BAD_ARG;
   const int drp = (dr + 31) & ~31;
-  const size_t smem = (size_t)(32 * (R + drp + 8) + R * 40) * sizeof(bf16_t);
+  const size_t smem = (size_t)(32 * (R + drp + 8) + R * 40 + 64 * (R + 8)) * sizeof(bf16_t);
   dim3 grid((unsigned)num_blocks);
   int rc;
 #define JLE_LATENT_LDS(NRV)                                                                                        \

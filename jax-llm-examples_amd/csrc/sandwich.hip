@@ -227,7 +227,7 @@ int launch_sandwich(const SandwichArgs& a, hipStream_t s) {
 
 // ------------------------------------------------------------------ polynomial activation
 // out = c0 N(u) + c1 N(u^2) + c2 N(u^3) + c3,  u = z + bias,  N(v) = v / sqrt(mean(v^2) + eps) over the row.
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(kThreads) void polynorm_kernel(const T* __restrict__ z, int ldz,
                                                             const float* __restrict__ bias,
                                                             const float* __restrict__ coef, float eps,
@@ -236,13 +236,17 @@ __global__ __launch_bounds__(kThreads) void polynorm_kernel(const T* __restrict_
   const size_t row = blockIdx.x;
   const T* zr = z + row * ldz;
   float s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  for (int d = threadIdx.x; d < F; d += kThreads) {
-    float u = Num<T>::load(zr + d);
-    if (bias != nullptr) u += bias[d];
-    const float u2 = u * u, u3 = u2 * u;
-    s1 = __builtin_fmaf(u, u, s1);
-    s2 = __builtin_fmaf(u2, u2, s2);
-    s3 = __builtin_fmaf(u3, u3, s3);
+  for (int d = threadIdx.x * VEC; d < F; d += kThreads * VEC) {
+    float u[VEC];
+    load_piece<T, VEC>(zr + d, u);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if (bias != nullptr) u[e] += bias[d + e];
+      const float u2 = u[e] * u[e], u3 = u2 * u[e];
+      s1 = __builtin_fmaf(u[e], u[e], s1);
+      s2 = __builtin_fmaf(u2, u2, s2);
+      s3 = __builtin_fmaf(u3, u3, s3);
+    }
   }
   const float t1 = block_sum<kThreads>(s1, red);
   const float t2 = block_sum<kThreads>(s2, red);
@@ -252,11 +256,16 @@ __global__ __launch_bounds__(kThreads) void polynorm_kernel(const T* __restrict_
   const float i3 = coef[2] / sqrtf(t3 / (float)F + eps);
   const float c3 = coef[3];
   T* o = out + row * F;
-  for (int d = threadIdx.x; d < F; d += kThreads) {
-    float u = Num<T>::load(zr + d);
-    if (bias != nullptr) u += bias[d];
-    const float u2 = u * u;
-    Num<T>::store(o + d, u * i1 + u2 * i2 + u2 * u * i3 + c3);
+  for (int d = threadIdx.x * VEC; d < F; d += kThreads * VEC) {
+    float u[VEC], v[VEC];
+    load_piece<T, VEC>(zr + d, u);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if (bias != nullptr) u[e] += bias[d + e];
+      const float u2 = u[e] * u[e];
+      v[e] = u[e] * i1 + u2 * i2 + u2 * u[e] * i3 + c3;
+    }
+    store_piece<T, VEC>(o + d, v);
   }
 }
 
@@ -296,12 +305,23 @@ JLE_API int jle_polynorm(const void* z, int ldz, const float* bias, const float*
                          int is_bf16, int N, int F, hipStream_t s) {
   if (N <= 0) return 0;
   if (F <= 0 || ldz < F || coef == nullptr) return JLE_BAD_ARG;
-  if (is_bf16)
-    hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(N), dim3(kThreads), 0, s, (const bf16_t*)z, ldz, bias, coef, eps,
-                       (bf16_t*)out, F);
-  else
-    hipLaunchKernelGGL(polynorm_kernel<float>, dim3(N), dim3(kThreads), 0, s, (const float*)z, ldz, bias, coef, eps,
-                       (float*)out, F);
+  // (which of the two forms runs depends on the width and on where the arrays lie, not on the step)
+  const bool vec = F % 4 == 0 && ldz % 4 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0;
+  if (is_bf16) {
+    if (vec)
+      hipLaunchKernelGGL((polynorm_kernel<bf16_t, 4>), dim3(N), dim3(kThreads), 0, s, (const bf16_t*)z, ldz, bias, coef,
+                         eps, (bf16_t*)out, F);
+    else
+      hipLaunchKernelGGL((polynorm_kernel<bf16_t, 1>), dim3(N), dim3(kThreads), 0, s, (const bf16_t*)z, ldz, bias, coef,
+                         eps, (bf16_t*)out, F);
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((polynorm_kernel<float, 4>), dim3(N), dim3(kThreads), 0, s, (const float*)z, ldz, bias, coef,
+                         eps, (float*)out, F);
+    else
+      hipLaunchKernelGGL((polynorm_kernel<float, 1>), dim3(N), dim3(kThreads), 0, s, (const float*)z, ldz, bias, coef,
+                         eps, (float*)out, F);
+  }
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -299,7 +299,7 @@ class HipOps:
 
     LATENT_SPLIT_BELOW = 2048  # fewer (token, head) pairs than this: a query's key tiles are shared between wavefronts
 
-    LATENT_MFMA_ITEMS = 1024  # the matrix-core kernel: fewer row tiles than this share their key steps between wavefronts
+    LATENT_MFMA_ITEMS = 512  # the matrix-core kernel: fewer row tiles than this share their key steps between wavefronts
     LATENT_LDS_TILES = 1024  # from so many row tiles on: the kernel whose blocks share keys through shared memory
 
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
