@@ -360,6 +360,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         ka[NR + c] = load16(krow + min(k0, dr - 8));
         if (!have || k0 >= dr) ka[NR + c] = zero4;
       }
+      __builtin_amdgcn_sched_barrier(0);  // (every load above is asked for before the first product below)
 #pragma unroll
       for (int c = 0; c < NR + 2; ++c)
         st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[c]), qb[c], st[t], 0, 0, 0);
@@ -407,11 +408,22 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
       for (int dt = 0; dt < NR * 2; ++dt) acc[dt] *= corr;
     }
 #pragma unroll
-    for (int dt = 0; dt < NR * 2; ++dt) {
-      u32x4 v = load16(vbase + (size_t)min(dt * 16, R - 16) * ps);
-      v &= keep;
-      if (dt * 16 >= R) v = zero4;
-      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, acc[dt], 0, 0, 0);
+    for (int d0 = 0; d0 < NR * 2; d0 += 16) {  // sixteen operands asked for together
+      u32x4 v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        if (d0 + u < NR * 2) {
+          v[u] = load16(vbase + (size_t)min((d0 + u) * 16, R - 16) * ps);
+          v[u] &= keep;
+          if ((d0 + u) * 16 >= R) v[u] = zero4;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (d0 + u < NR * 2)
+          acc[d0 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v[u]), pb, acc[d0 + u], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   if (!row_ok) return;
@@ -743,6 +755,30 @@ JLE_API int jle_latent_attention_mfma(const void* q_lat, const void* q, int q_ld
     hipLaunchKernelGGL(latent_attention_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * H, R, splits);
     JLE_LAUNCH_CHECK();
   }
+  return 0;
+}
+
+// out[b][a][:] = in[a][b][:] for rows of row_bytes bytes (a multiple of 4; of 16 where the arrays allow it).
+__global__ __launch_bounds__(256) void swap_leading_kernel(const uint32_t* __restrict__ in, uint32_t* __restrict__ out,
+                                                           int A, int B, int words) {
+  const size_t pair = blockIdx.x;  // = b * A + a
+  const int b = (int)(pair / A), a = (int)(pair - (size_t)b * A);
+  const uint32_t* src = in + ((size_t)a * B + b) * words;
+  uint32_t* dst = out + pair * words;
+  if (words % 4 == 0 && ((uintptr_t)in | (uintptr_t)out) % 16 == 0) {
+    for (int i = threadIdx.x * 4; i < words; i += 256 * 4)
+      *reinterpret_cast<uint4*>(dst + i) = *reinterpret_cast<const uint4*>(src + i);
+  } else {
+    for (int i = threadIdx.x; i < words; i += 256) dst[i] = src[i];
+  }
+}
+
+JLE_API int jle_swap_leading(const void* in, void* out, int A, int B, int row_bytes, hipStream_t s) {
+  if (A <= 0 || B <= 0) return 0;
+  if (row_bytes <= 0 || row_bytes % 4 || (long long)A * B > (1ll << 31) - 1) return JLE_BAD_ARG;
+  hipLaunchKernelGGL(swap_leading_kernel, dim3((unsigned)((long long)A * B)), dim3(256), 0, s, (const uint32_t*)in,
+                     (uint32_t*)out, A, B, row_bytes / 4);
+  JLE_LAUNCH_CHECK();
   return 0;
 }
 

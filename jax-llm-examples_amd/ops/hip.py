@@ -61,6 +61,7 @@ _SIGNATURES = {
                            _vp, _i, _i, _i, _i, _vp],
     "jle_polynorm": [_vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
     "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
+    "jle_swap_leading": [_vp, _vp, _i, _i, _i, _vp],
     "jle_latent_attention_lds": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
                                  _i, _i, _vp],
     "jle_latent_attention_mfma": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
@@ -267,7 +268,15 @@ class HipOps:
         """``out[b] = a[b] @ w[b]`` for ``a [B, N, K]``, ``w [B, K, M]`` (views with any strides): a library
         product, true float32 in float32.  ``[B, N, M]``, or with ``tokens_first`` laid out ``[N, B, M]``."""
         out = torch.bmm(a, w)
-        return out.transpose(0, 1).contiguous() if tokens_first else out
+        if not tokens_first:
+            return out
+        b, n, m = out.shape
+        row_bytes = m * out.element_size()
+        if row_bytes % 4 or not out.is_contiguous():
+            return out.transpose(0, 1).contiguous()
+        swapped = torch.empty(n, b, m, dtype=out.dtype, device=out.device)
+        self._call("jle_swap_leading", _p(out), _p(swapped), b, n, row_bytes)
+        return swapped
 
     def latent_prepare(self, rows, num_heads: int, nope_dim: int, rope_dim: int, kv_rank: int, positions, rotation,
                        latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool,
