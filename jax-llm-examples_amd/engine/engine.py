@@ -38,7 +38,8 @@ class Engine:
         ``decode_graphs``: replay steps of single tokens as recorded HIP graphs (default: on a GPU)."""
         self.model = model
         self.max_num_batched_tokens = max_num_batched_tokens
-        self.ops = get_ops(model.device, reference_ops=reference_ops)
+        self.ops = get_ops(model.device, reference_ops=reference_ops,
+                           kernel_sources=getattr(getattr(model, "arch", None), "kernel_sources", None))
         limit = getattr(getattr(model, "config", None), "max_position_embeddings", None)
         asked_len = max_seq_len
         if max_seq_len is None:

@@ -27,7 +27,7 @@ def parse_dtype(name) -> torch.dtype:
         raise ValueError(f"run dtype must be bfloat16 or float32, got {name!r}") from None
 
 
-def get_ops(device, reference_ops: bool = False):
+def get_ops(device, reference_ops: bool = False, kernel_sources=None):
     """The kernel set for ``device``.  On a GPU that is the compiled HIP library
     (an error if it cannot be built or loaded: there is no fallback).  The plain
     PyTorch ops are handed out only when asked for by name, for tests of the
@@ -44,7 +44,9 @@ def get_ops(device, reference_ops: bool = False):
         )
     from ..ops.hip import HipOps
 
-    return HipOps(device)
+    # (``kernel_sources``: what the model's architecture says it needs of ``csrc/``; if no library is built yet,
+    # only that is compiled now)
+    return HipOps(device, kernel_sources=kernel_sources)
 
 
 def build_model(arch, cfg, dtype, device) -> DecoderModel:

@@ -22,6 +22,7 @@ import sys
 import torch
 
 from ..cache.manager import CacheManager
+from ..config.registry import architecture_name, get_architecture, read_config_json
 from .batch import StepEntry
 from .loading import get_ops, load_model, parse_dtype
 from .runner import ModelRunner
@@ -34,7 +35,8 @@ def make_runner(model_dir: str, dtype, max_tokens: int, device: str = "cuda:0", 
     counts that are rounded to pages here), so pages are used again.  ``max_requests``: requests
     that may be live at once."""
     dtype = parse_dtype(dtype)
-    ops = get_ops(device, reference_ops=reference_ops)
+    arch = get_architecture(architecture_name(read_config_json(model_dir)))
+    ops = get_ops(device, reference_ops=reference_ops, kernel_sources=getattr(arch, "kernel_sources", None))
     model = load_model(model_dir, dtype, device)
     rounded = -(-max_tokens // 64) * 64
     num_pages = -(-rounded // page_size) + max_requests

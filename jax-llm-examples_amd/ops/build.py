@@ -35,9 +35,10 @@ def _headers() -> list[str]:
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
 
 
-def source_hash() -> str:
+def source_hash(only=None) -> str:
+    """``only``: a subset of the sources (a library of those alone has a name of its own)."""
     h = hashlib.sha256()
-    for name in sources() + _headers():
+    for name in (sorted(only) if only else sources()) + _headers():
         h.update(name.encode())
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
@@ -73,8 +74,13 @@ def _say(msg: str) -> None:
     print(f"[jle build] {msg}", file=sys.stderr, flush=True)
 
 
-def find_library() -> str | None:
-    name = f"libjle-{source_hash()}.so"
+def _library_name(only=None) -> str:
+    return f"libjle-part-{source_hash(only)}.so" if only else f"libjle-{source_hash()}.so"
+
+
+def find_library(only=None) -> str | None:
+    """The built library of all sources, or (``only``) of a subset of them."""
+    name = _library_name(only)
     for d in (os.environ.get("JLE_BUILD_DIR"), os.path.join(CSRC, "_build"),
               os.path.join(tempfile.gettempdir(), f"jle-build-{os.getuid()}")):
         if d and os.path.exists(os.path.join(d, name)):
@@ -82,17 +88,23 @@ def find_library() -> str | None:
     return None
 
 
-def build(force: bool = False, jobs: int | None = None) -> str:
+def build(force: bool = False, jobs: int | None = None, only=None) -> str:
+    """``only``: compile and link just these sources (what one kind of model needs): a library of its own, which
+    lacks the other sources' entry points."""
+    if only:
+        unknown = sorted(set(only) - set(sources()))
+        if unknown:
+            raise RuntimeError(f"no such kernel source(s): {', '.join(unknown)}")
     if not force:
-        found = find_library()
+        found = find_library(only)
         if found:
             return found
     hipcc = _hipcc()
     out_dir = _build_dir()
-    tag = source_hash()
+    tag = source_hash(only)
     obj_dir = os.path.join(out_dir, f"obj-{tag}-{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
-    srcs = sources()
+    srcs = sorted(only) if only else sources()
     jobs = jobs or min(len(srcs), max(1, min(16, os.cpu_count() or 4)))
     _say(f"compiling {len(srcs)} HIP sources for {ARCH} with {jobs} jobs (first use; this takes a minute or two)")
     t0 = time.time()
@@ -114,7 +126,7 @@ def build(force: bool = False, jobs: int | None = None) -> str:
             for f in done:
                 objs.append(f.result())
             _say(f"{len(srcs) - len(pending)}/{len(srcs)} sources compiled after {time.time() - t0:.0f} s")
-    lib = os.path.join(out_dir, f"libjle-{tag}.so")
+    lib = os.path.join(out_dir, _library_name(only))
     tmp = lib + f".tmp{os.getpid()}"
     r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *sorted(objs), "-o", tmp],
                        capture_output=True, text=True)
@@ -122,8 +134,9 @@ def build(force: bool = False, jobs: int | None = None) -> str:
         raise RuntimeError(f"linking the kernel library failed:\n{r.stdout}\n{r.stderr}")
     os.replace(tmp, lib)
     shutil.rmtree(obj_dir, ignore_errors=True)
-    for f in os.listdir(out_dir):  # older builds
-        if f.startswith("libjle-") and f.endswith(".so") and f != os.path.basename(lib):
+    for f in os.listdir(out_dir):  # older builds of the same kind
+        if (f.startswith("libjle-") and f.endswith(".so") and f != os.path.basename(lib)
+                and f.startswith("libjle-part-") == bool(only)):
             try:
                 os.remove(os.path.join(out_dir, f))
             except OSError:
@@ -132,5 +145,9 @@ def build(force: bool = False, jobs: int | None = None) -> str:
     return lib
 
 
-def library_path() -> str:
+def library_path(only=None) -> str:
+    """The library of all sources if it is built; else, with ``only``, the library of that subset (built if it is
+    not there); else the library of all sources, built now."""
+    if only:
+        return find_library() or build(force=False, only=only)
     return build(force=False)

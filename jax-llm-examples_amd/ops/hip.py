@@ -117,26 +117,34 @@ class PendingNorm:
 _LIB = None
 
 
-def load_library():
-    """Loads the compiled kernels (compiling them if no build is there)."""
-    global _LIB
-    if _LIB is None:
-        path = _build.library_path()
-        try:
-            lib = ctypes.CDLL(path)
-        except OSError as e:
-            raise KernelError(f"cannot load the HIP kernel library {path}: {e}") from e
-        for name, args in _SIGNATURES.items():
-            fn = getattr(lib, name)
+def _bind(path: str):
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelError(f"cannot load the HIP kernel library {path}: {e}") from e
+    for name, args in _SIGNATURES.items():
+        fn = getattr(lib, name, None)  # (a library of some of the sources lacks the others' entry points)
+        if fn is not None:
             fn.argtypes = args
             fn.restype = ctypes.c_int
-        lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
-        lib.jle_gemm_stream_supported.argtypes = [_i, _i, _i]
-        lib.jle_latent_attention_mfma_supported.argtypes = [_i, _i, _i, _i, _i]
-        lib.jle_gemm_f32_stream_supported.argtypes = [_i, _i, _i]
-        lib.jle_attention_group_waves.argtypes = []
-        lib._jle_path = path
-        _LIB = lib
+    for name, args in (("jle_attention_mfma_supported", [_i, _i, _i, _i]),  # queries, not launches: no stream
+                       ("jle_gemm_stream_supported", [_i, _i, _i]), ("jle_gemm_f32_stream_supported", [_i, _i, _i]),
+                       ("jle_latent_attention_mfma_supported", [_i, _i, _i, _i, _i]), ("jle_attention_group_waves", [])):
+        fn = getattr(lib, name, None)
+        if fn is not None:
+            fn.argtypes = args
+    lib._jle_path = path
+    lib._jle_whole = "libjle-part-" not in path
+    return lib
+
+
+def load_library(kernel_sources=None):
+    """Loads the compiled kernels (compiling them if no build is there).  ``kernel_sources``: the sources that the
+    model to be run needs; if the library of all sources is not built yet, only those are compiled now.  A kernel
+    that such a library lacks and that is called all the same brings the whole library in (:meth:`HipOps._whole`)."""
+    global _LIB
+    if _LIB is None:
+        _LIB = _bind(_build.library_path(only=kernel_sources))
     return _LIB
 
 
@@ -147,12 +155,12 @@ def _p(t: Optional[torch.Tensor]):
 class HipOps:
     name = "hip"
 
-    def __init__(self, device) -> None:
+    def __init__(self, device, kernel_sources=None) -> None:
         self.device = torch.device(device)
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise KernelError("the HIP kernels need a GPU")
-        self.lib = load_library()
-        self._fn = {name: getattr(self.lib, name) for name in _SIGNATURES}
+        self.lib = load_library(kernel_sources)
+        self._fn = {name: getattr(self.lib, name) for name in _SIGNATURES if hasattr(self.lib, name)}
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._raw_stream = raw if raw is not None else (lambda i: torch.cuda.current_stream(i).cuda_stream)
@@ -171,7 +179,23 @@ class HipOps:
         """The current stream's handle (a decode step asks hundreds of times: the raw query, not a Stream object)."""
         return self._raw_stream(self._device_index)
 
+    def _whole(self) -> None:
+        """The library of all sources instead of the partial one this process began with (built now if need be)."""
+        global _LIB
+        if not self.lib._jle_whole:
+            _LIB = _bind(_build.library_path())
+        self.lib = _LIB
+        self._fn = {name: getattr(self.lib, name) for name in _SIGNATURES}
+
+    def _query(self, name: str, *args) -> int:
+        """An entry point that answers a question about sizes (no launch, no stream)."""
+        if not hasattr(self.lib, name):
+            self._whole()
+        return getattr(self.lib, name)(*args)
+
     def _call(self, name: str, *args) -> None:
+        if name not in self._fn:
+            self._whole()
         rc = self._fn[name](*args, self._stream())
         if rc != 0:
             if rc < 0:
@@ -331,7 +355,7 @@ class HipOps:
         w = 0 if window is None else int(window)
         out = torch.empty(n, H, r, dtype=q_lat.dtype, device=q_lat.device)
         if (latent_t_pages is not None and q_lat.dtype == torch.bfloat16
-                and self.lib.jle_latent_attention_mfma_supported(r, nope_dim, dr, q_ld, ps)):
+                and self._query("jle_latent_attention_mfma_supported", r, nope_dim, dr, q_ld, ps)):
             self._chk(latent_t_pages, latent_pages.dtype, (np_, ps, r), "transposed latent pages")
             return self._latent_attention_mfma(q_lat, q, q_ld, nope_dim, dr, latent_pages, latent_t_pages, rope_pages,
                                                out, block_table, positions, token_segment, w, scale, meta)
@@ -540,7 +564,7 @@ class HipOps:
         return out
 
     def f32_stream_supported(self, nout: int, k: int, swiglu: bool) -> bool:
-        return bool(self.lib.jle_gemm_f32_stream_supported(nout, k, int(swiglu)))
+        return bool(self._query("jle_gemm_f32_stream_supported", nout, k, int(swiglu)))
 
     def gemm_f32_stream(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, rows=None):
         """The float32 grouped product for about a hundred rows per group on the float32 matrix instructions,
@@ -653,7 +677,7 @@ class HipOps:
 
 
     def stream_supported(self, nout: int, k: int, swiglu: bool) -> bool:
-        return bool(self.lib.jle_gemm_stream_supported(nout, k, int(swiglu)))
+        return bool(self._query("jle_gemm_stream_supported", nout, k, int(swiglu)))
 
     def gemm_stream(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None):
         """bfloat16 product on MFMA for about a hundred rows per group, weights in the streaming layout and
@@ -750,7 +774,7 @@ class HipOps:
         group = hq // max(hk, 1)
         if (meta is not None and meta.decode_bucket is not None and qkv.dtype == torch.bfloat16 and prep.plain
                 and group <= 32 and n * hk < self.TICKETS and 4 * (dh + 4 * group * (dh + 2)) <= 48 * 1024
-                and self.lib.jle_attention_mfma_supported(dh, hq, hk, ps)):
+                and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
             self._chk(qkv, kv_cache.dtype, (n, (hq + 2 * hk) * dh), "q|k|v")
             self._chk(kv_cache, None, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")
             self._chk(block_table, torch.int32, None, "block table")
@@ -856,7 +880,7 @@ class HipOps:
         groups = []
         if tiles and group_size > 1 and self.PREFILL_TILE == 32:
             # consecutive (tile, head) items of one segment, `waves` per block; blocks with the most keys first
-            waves = int(self.lib.jle_attention_group_waves())
+            waves = int(self._query("jle_attention_group_waves"))
             keyed = []
             for first, count, last_pos in seg_tiles:
                 items = count * group_size
@@ -905,7 +929,7 @@ class HipOps:
         param = int(retention[1]) if len(retention) > 1 else 0
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
         if (q.dtype == torch.bfloat16 and hq // hk <= 32
-                and self.lib.jle_attention_mfma_supported(dh, hq, hk, ps)):
+                and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
             key = f"attn_plan_{hq // hk}"
             plan = meta.meta.get(key) if meta is not None else None
             if plan is None:

@@ -20,6 +20,9 @@ from ..weights.bindings import TensorBinding
 
 class RovidraArchitecture:
     names = ("Rovidra", "rovidra")
+    # what of csrc/ a model of this design calls (a first run on a machine without a built library compiles these)
+    kernel_sources = ("elementwise.hip", "sandwich.hip", "attention_latent.hip", "gemm_skinny.hip", "gemm_stream.hip",
+                      "gemm_grouped.hip", "gemm_generic.hip", "sampling.hip")
 
     def parse_config(self, top: Mapping[str, Any]) -> RovidraConfig:
         return RovidraConfig.from_dict(top)

@@ -413,6 +413,19 @@ def test_greedy_generation_in_bfloat16(folders_bf16):
 
 
 @pytest.mark.gpu
+def test_command_line(folders, capsys):
+    """``python -m jax_llm_examples_amd.main`` picks the design by config.json like every other entry point."""
+    from jax_llm_examples_amd.main import main
+
+    plain = P.PlainRovidra(folders["RA"])
+    rc = main(["--ckpt-path", folders["RA"], "--dtype", "float32", "--prompt-ids", "5,6,7,8", "--prompt-ids", "9",
+               "--max-decode-length", "6", "--decode-batch-size", "2", "--max-seq-len", "64"])
+    assert rc == 0
+    lines = [json.loads(ln) for ln in capsys.readouterr().out.strip().splitlines()]
+    assert [ln["tokens"] for ln in lines] == [_greedy(plain, [5, 6, 7, 8], 6), _greedy(plain, [9], 6)]
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(folders_bf16, tmp_path, dtype):
     """``bin/trace_run`` as a program, on a folder that holds config.json and bfloat16 weights."""
@@ -438,6 +451,40 @@ def test_trace_run_program(folders_bf16, tmp_path, dtype):
                 assert float((torch.from_numpy(got[o].copy()) - r).abs().max() / ref[e["id"]].abs().max()) < TOL[dtype]
                 o += 1
             at[e["id"]] += len(e["tokens"])
+
+
+@pytest.mark.gpu
+def test_library_of_the_designs_own_sources(folders, tmp_path):
+    """A process that starts with the library of only the sources this design names runs the design, and brings the
+    whole library in when another model calls a kernel that the partial one lacks."""
+    from jax_llm_examples_amd.ops import build
+
+    arch = get_architecture("Rovidra")
+    partial = build.find_library(only=arch.kernel_sources)
+    if partial is None or build.find_library() is None:
+        pytest.skip("the partial kernel library is not built in this tree")
+    code = f"""
+import sys, torch
+sys.path.insert(0, {ROOT!r}); sys.path.insert(0, {os.path.join(ROOT, 'tests')!r})
+from jax_llm_examples_amd.ops import hip
+hip._LIB = hip._bind({partial!r})
+assert not hip._LIB._jle_whole and not hasattr(hip._LIB, "jle_moe_route")
+from jax_llm_examples_amd.engine.replay import make_runner
+from jax_llm_examples_amd.engine import StepEntry
+import plain_rovidra as P
+toks = [5, 9, 200, 31, 7, 7, 100, 3]
+runner = make_runner({folders['RA']!r}, "float32", 64, "cuda:0", max_requests=2)
+got = runner.step([StepEntry("r", toks, list(range(len(toks))))]).cpu()
+ref = P.PlainRovidra({folders['RA']!r}).logits(toks).float()
+assert float((got - ref).abs().max() / ref.abs().max()) < 2e-5
+assert not runner.ops.lib._jle_whole
+x = torch.randn(4, 64, device="cuda:0"); r = torch.randn(8, 64, device="cuda:0")
+ids, gates = runner.ops.moe_route(x, r, 1)  # a kernel of another source
+assert runner.ops.lib._jle_whole and ids.shape == (4, 1)
+print("ok")
+"""
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("ok"), proc.stderr[-2000:]
 
 
 # ---------------------------------------------------------------------------------------------- configuration, weights
