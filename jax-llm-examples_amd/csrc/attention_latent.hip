@@ -576,35 +576,39 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
     __syncthreads();
     if (t0 + 32 <= bhi) prefetch(t0 + 32);
     if (!active || t0 + 31 < lo || t0 > hi) continue;  // none of this tile's rows sees a key of the step
-    f32x4 st[2];
+    // (no branch in these loops: reads on the far side of a branch are not asked for before the products on this
+    // side are done; a chunk past the latent's width is a product with zeros.  A chunk of the queries is read once
+    // for both key tiles.)
+    f32x4 st[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    const bf16_t* arow0 = sk + r * KS + g * 8;
+    const bf16_t* arow1 = arow0 + 16 * KS;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* arow = sk + (16 * t + r) * KS + g * 8;
-      // (no branch in these loops: reads on the far side of a branch are not asked for before the products on this
-      // side are done; a chunk past the latent's width is a product with zeros)
+    for (int c0 = 0; c0 < NR; c0 += 2) {  // two chunks' reads under way at a time, no more: registers
+      u32x4 a0[2], a1[2], b[2];
 #pragma unroll
-      for (int c0 = 0; c0 < NR; c0 += 2) {  // two chunks' reads under way at a time, no more: registers
-        u32x4 a[2], b[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int c = c0 + u;
-          a[u] = load16(arow + min(c * 32, R - 32));
-          b[u] = load16(qrow + min(c * 32, R - 32));
-          if (c * 32 >= R) a[u] = zero4;
-        }
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-          st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]),
-                                                          __builtin_bit_cast(bf16x8, b[u]), st[t], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int u = 0; u < 2; ++u) {
+        const int off = min((c0 + u) * 32, R - 32);
+        a0[u] = load16(arow0 + off);
+        a1[u] = load16(arow1 + off);
+        b[u] = load16(qrow + off);
+        if ((c0 + u) * 32 >= R) b[u] = zero4;
       }
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        u32x4 a = load16(arow + R + min(c * 32, drp - 32));
-        if (c * 32 >= drp) a = zero4;
-        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qrot[c], st[t], 0, 0, 0);
+      for (int u = 0; u < 2; ++u) {
+        st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a0[u]),
+                                                        __builtin_bit_cast(bf16x8, b[u]), st[0], 0, 0, 0);
+        st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a1[u]),
+                                                        __builtin_bit_cast(bf16x8, b[u]), st[1], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int off = R + min(c * 32, drp - 32);
+      u32x4 a0 = load16(arow0 + off), a1 = load16(arow1 + off);
+      if (c * 32 >= drp) a0 = a1 = zero4;
+      st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a0), qrot[c], st[0], 0, 0, 0);
+      st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a1), qrot[c], st[1], 0, 0, 0);
     }
     float sv8[8];
     float mx = -INFINITY;

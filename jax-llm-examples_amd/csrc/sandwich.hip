@@ -227,7 +227,9 @@ int launch_sandwich(const SandwichArgs& a, hipStream_t s) {
 
 // ------------------------------------------------------------------ polynomial activation
 // out = c0 N(u) + c1 N(u^2) + c2 N(u^3) + c3,  u = z + bias,  N(v) = v / sqrt(mean(v^2) + eps) over the row.
-template <typename T, int VEC>
+// PIECES > 0: the row (up to kThreads * VEC * PIECES wide) stays in registers between the sums and the polynomial;
+// PIECES == 0: any width, the row is read twice.
+template <typename T, int VEC, int PIECES>
 __global__ __launch_bounds__(kThreads) void polynorm_kernel(const T* __restrict__ z, int ldz,
                                                             const float* __restrict__ bias,
                                                             const float* __restrict__ coef, float eps,
@@ -235,17 +237,41 @@ __global__ __launch_bounds__(kThreads) void polynorm_kernel(const T* __restrict_
   __shared__ float red[kThreads / 64];
   const size_t row = blockIdx.x;
   const T* zr = z + row * ldz;
+  T* o = out + row * F;
   float s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  for (int d = threadIdx.x * VEC; d < F; d += kThreads * VEC) {
-    float u[VEC];
-    load_piece<T, VEC>(zr + d, u);
+  auto sums = [&](const float (&u)[VEC]) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-      if (bias != nullptr) u[e] += bias[d + e];
       const float u2 = u[e] * u[e], u3 = u2 * u[e];
       s1 = __builtin_fmaf(u[e], u[e], s1);
       s2 = __builtin_fmaf(u2, u2, s2);
       s3 = __builtin_fmaf(u3, u3, s3);
+    }
+  };
+  auto fetch = [&](int d, float (&u)[VEC]) {
+    load_piece<T, VEC>(zr + d, u);
+    if (bias != nullptr) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) u[e] += bias[d + e];
+    }
+  };
+  constexpr int P = PIECES > 0 ? PIECES : 1;
+  float kept[P][VEC];
+  if constexpr (PIECES > 0) {
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int d = (threadIdx.x + kThreads * i) * VEC;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) kept[i][e] = 0.f;
+      if (d < F) fetch(d, kept[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) sums(kept[i]);  // (zeros beyond the row's end add nothing)
+  } else {
+    for (int d = threadIdx.x * VEC; d < F; d += kThreads * VEC) {
+      float u[VEC];
+      fetch(d, u);
+      sums(u);
     }
   }
   const float t1 = block_sum<kThreads>(s1, red);
@@ -255,18 +281,47 @@ __global__ __launch_bounds__(kThreads) void polynorm_kernel(const T* __restrict_
   const float i2 = coef[1] / sqrtf(t2 / (float)F + eps);
   const float i3 = coef[2] / sqrtf(t3 / (float)F + eps);
   const float c3 = coef[3];
-  T* o = out + row * F;
-  for (int d = threadIdx.x * VEC; d < F; d += kThreads * VEC) {
-    float u[VEC], v[VEC];
-    load_piece<T, VEC>(zr + d, u);
+  auto poly = [&](const float (&u)[VEC], float (&v)[VEC]) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-      if (bias != nullptr) u[e] += bias[d + e];
       const float u2 = u[e] * u[e];
       v[e] = u[e] * i1 + u2 * i2 + u2 * u[e] * i3 + c3;
     }
-    store_piece<T, VEC>(o + d, v);
+  };
+  if constexpr (PIECES > 0) {
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int d = (threadIdx.x + kThreads * i) * VEC;
+      if (d < F) {
+        float v[VEC];
+        poly(kept[i], v);
+        store_piece<T, VEC>(o + d, v);
+      }
+    }
+  } else {
+    for (int d = threadIdx.x * VEC; d < F; d += kThreads * VEC) {
+      float u[VEC], v[VEC];
+      fetch(d, u);
+      poly(u, v);
+      store_piece<T, VEC>(o + d, v);
+    }
   }
+}
+
+template <typename T>
+void launch_polynorm(const T* z, int ldz, const float* bias, const float* coef, float eps, T* out, int N, int F,
+                     bool vec, hipStream_t s) {
+  // (which form runs depends on the width and on where the arrays lie, not on the step; the sums of a row are
+  // formed in the same order in the forms that keep the row and in the one that reads it twice)
+  dim3 g(N), b(kThreads);
+  if (vec && F <= kThreads * 4 * 4)
+    hipLaunchKernelGGL((polynorm_kernel<T, 4, 4>), g, b, 0, s, z, ldz, bias, coef, eps, out, F);
+  else if (vec && F <= kThreads * 4 * 16)
+    hipLaunchKernelGGL((polynorm_kernel<T, 4, 16>), g, b, 0, s, z, ldz, bias, coef, eps, out, F);
+  else if (vec)
+    hipLaunchKernelGGL((polynorm_kernel<T, 4, 0>), g, b, 0, s, z, ldz, bias, coef, eps, out, F);
+  else
+    hipLaunchKernelGGL((polynorm_kernel<T, 1, 0>), g, b, 0, s, z, ldz, bias, coef, eps, out, F);
 }
 
 }  // namespace
@@ -305,23 +360,11 @@ JLE_API int jle_polynorm(const void* z, int ldz, const float* bias, const float*
                          int is_bf16, int N, int F, hipStream_t s) {
   if (N <= 0) return 0;
   if (F <= 0 || ldz < F || coef == nullptr) return JLE_BAD_ARG;
-  // (which of the two forms runs depends on the width and on where the arrays lie, not on the step)
   const bool vec = F % 4 == 0 && ldz % 4 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0;
-  if (is_bf16) {
-    if (vec)
-      hipLaunchKernelGGL((polynorm_kernel<bf16_t, 4>), dim3(N), dim3(kThreads), 0, s, (const bf16_t*)z, ldz, bias, coef,
-                         eps, (bf16_t*)out, F);
-    else
-      hipLaunchKernelGGL((polynorm_kernel<bf16_t, 1>), dim3(N), dim3(kThreads), 0, s, (const bf16_t*)z, ldz, bias, coef,
-                         eps, (bf16_t*)out, F);
-  } else {
-    if (vec)
-      hipLaunchKernelGGL((polynorm_kernel<float, 4>), dim3(N), dim3(kThreads), 0, s, (const float*)z, ldz, bias, coef,
-                         eps, (float*)out, F);
-    else
-      hipLaunchKernelGGL((polynorm_kernel<float, 1>), dim3(N), dim3(kThreads), 0, s, (const float*)z, ldz, bias, coef,
-                         eps, (float*)out, F);
-  }
+  if (is_bf16)
+    launch_polynorm<bf16_t>((const bf16_t*)z, ldz, bias, coef, eps, (bf16_t*)out, N, F, vec, s);
+  else
+    launch_polynorm<float>((const float*)z, ldz, bias, coef, eps, (float*)out, N, F, vec, s);
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -231,8 +231,8 @@ class HipOps:
         self._call("jle_embed", _p(token_ids), _p(table), self._is_bf16(table), _p(out), n, d)
         return out
 
-    SHIFT_ROWS_PER_BLOCK = 8  # a block of the norm-and-shift kernel takes so many rows in a step of many tokens
-    # (it forms the row before its first anew)
+    SHIFT_ROWS_PER_BLOCK = 4  # a block of the norm-and-shift kernel takes so many rows in a step of many tokens
+    # (it forms the row before its first anew: with one row a block every row is formed twice)
 
     def add_norm_shift(self, x, delta, weight, eps: float, out_dtype, shift, ctx, do_norm: bool = True):
         """``x' = x + delta`` into a new tensor (``delta``: ``None``, a tensor, or a gated branch
@@ -265,7 +265,7 @@ class HipOps:
             self._chk(sw, torch.float32, (d,), "shift weight")
             self._chk(state, torch.float32, (state.shape[0], 2, d), "shift state")
             hs = torch.empty(n, d, dtype=out_dtype, device=x.device)
-            rows = self.SHIFT_ROWS_PER_BLOCK if n >= 4 * self._compute_units * self.SHIFT_ROWS_PER_BLOCK else 1
+            rows = self.SHIFT_ROWS_PER_BLOCK if n >= self._compute_units * self.SHIFT_ROWS_PER_BLOCK else 1
         is_bf16 = 1 if out_dtype == torch.bfloat16 else 0
         self._call("jle_add_norm_shift", _p(x), _p(x_out), kind, _p(y), _p(yb), _p(g), _p(gb), _p(pw), float(peps),
                    int(do_norm), _p(weight), float(eps), _p(h), _p(sw), _p(hs), _p(state),
