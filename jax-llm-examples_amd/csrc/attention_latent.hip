@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ row
   for (int d = rd + threadIdx.x; d < dr; d += 256) rp[d] = kr[d];  // what does not turn
 }
 
-constexpr int kMaxAcc = 8;  // latent elements per lane: kv_rank up to 512
+constexpr int kMaxAcc = 16;  // latent elements per lane: kv_rank up to 1024
 
 template <typename T>
 __global__ __launch_bounds__(256) void latent_attention_kernel(
