@@ -21,11 +21,6 @@ namespace {
 constexpr int kThreads = 256;
 
 template <typename T, int VEC>
-struct Piece {
-  float v[VEC];
-};
-
-template <typename T, int VEC>
 __device__ __forceinline__ void load_piece(const T* p, float (&o)[VEC]) {
   if constexpr (VEC == 4) {
     const f32x4_t r = load4<T>(p);

@@ -332,7 +332,9 @@ class HipOps:
 
     LATENT_SPLIT_BELOW = 2048  # fewer (token, head) pairs than this: a query's key tiles are shared between wavefronts
 
-    LATENT_MFMA_ITEMS = 512  # the matrix-core kernel: fewer row tiles than this share their key steps between wavefronts
+    LATENT_MFMA_ITEMS = 1024  # the matrix-core kernel: fewer row tiles than this share their key steps between
+    # wavefronts, about so many work items in all (measured at 256 / 512 / 1,024 / 2,048: batch 64 at 2,048 tokens of
+    # context 296 / 168 / 117 / 130 us a layer, batch 16 80 / 58 / 48 / 63)
     LATENT_LDS_TILES = 1024  # from so many row tiles on: the kernel whose blocks share keys through shared memory
 
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
