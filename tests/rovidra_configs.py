@@ -63,6 +63,18 @@ ROVIDRA_FAST = {
             _layer(_mixer(4, 64, 32, 64, 64, 0.1, 10000.0, mask=300), ff=512),
         ],
     },
+    # latents and rotated parts that fill no whole chunk of the matrix-core kernels (96 and 160 wide, 24 and 40
+    # rotated elements), 20 heads (a tile of 16 rows runs over two tokens), 6 heads, a window of one token
+    "RG": {
+        "seed": 13, "architecture": "Rovidra", "vocab": 777, "width": 192, "embedding": {"scale": 9.0},
+        "norm": {"eps": 1e-6},
+        "layers": [
+            _layer(_mixer(20, 16, 24, 8, 96, 0.2, 30000.0, dims=16, mask=45), ff=320),
+            _layer(_mixer(6, 40, 24, 24, 96, 0.18, 30000.0, dims=16, mask=1, kv_from=0)),
+            _layer(_mixer(3, 8, 40, 16, 160, 0.15, 777.0, mask=130), ff=200),
+            _layer(_mixer(17, 24, 40, 8, 160, 0.15, 777.0, kv_from=2), ff=64),
+        ],
+    },
 }
 
 

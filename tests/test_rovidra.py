@@ -29,7 +29,7 @@ from rovidra_configs import ROVIDRA, ROVIDRA_FAST, rovidra_config_json, write_ro
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DEVICES = [pytest.param("cpu", id="cpu-plain-ops"), pytest.param("cuda:0", id="gpu-hip", marks=pytest.mark.gpu)]
-LENGTHS = {"RA": [1, 80, 33, 47, 64, 9, 130], "RB": [70, 2, 49, 96, 31, 17], "RS": [61, 40, 5, 83], "RF": [420, 40, 170, 33]}
+LENGTHS = {"RA": [1, 80, 33, 47, 64, 9, 130], "RB": [70, 2, 49, 96, 31, 17], "RS": [61, 40, 5, 83], "RF": [420, 40, 170, 33], "RG": [150, 2, 61, 33, 97]}
 MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
 TOL = {"float32": 2e-5, "bfloat16": 3e-2}  # of the largest logit of the request
 # (bfloat16 with the sharp scores of RS: a rounding of a score of 40 by 2^-9 moves its weight by a tenth)
@@ -297,7 +297,7 @@ def test_gpu_bfloat16(folders_bf16, name, mode):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
-@pytest.mark.parametrize("name", ["RA", "RF"])
+@pytest.mark.parametrize("name", ["RA", "RF", "RG"])
 def test_gpu_bfloat16_with_keys_shared_through_shared_memory(folders_bf16, monkeypatch, name, mode):
     """Steps of many tokens go through the attention kernel whose blocks share their keys; here every step of more
     than a few rows does (tiles of several tokens, blocks that end inside a segment, windows that start inside a
