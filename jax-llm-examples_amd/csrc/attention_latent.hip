@@ -641,18 +641,29 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
 #pragma unroll
       for (int dt = 0; dt < NR * 2; ++dt) acc[dt] *= corr;
     }
+    // four operands are read while the four before them are multiplied
+    u32x4 vcur[4], vnext[4];
 #pragma unroll
-    for (int d0 = 0; d0 < NR * 2; d0 += 4) {  // four operands under way at a time
-      u32x4 v[4];
+    for (int u = 0; u < 4; ++u) {
+      vcur[u] = load16(vrow + min(u * 16, R - 16) * VS);
+      if (u * 16 >= R) vcur[u] = zero4;
+    }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        v[u] = load16(vrow + min((d0 + u) * 16, R - 16) * VS);
-        if ((d0 + u) * 16 >= R) v[u] = zero4;
+    for (int d0 = 0; d0 < NR * 2; d0 += 4) {
+      if (d0 + 4 < NR * 2) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          vnext[u] = load16(vrow + min((d0 + 4 + u) * 16, R - 16) * VS);
+          if ((d0 + 4 + u) * 16 >= R) vnext[u] = zero4;
+        }
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        acc[d0 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v[u]), pb, acc[d0 + u], 0, 0, 0);
+        acc[d0 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vcur[u]), pb, acc[d0 + u], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) vcur[u] = vnext[u];
     }
   }
   if (!row_ok) return;

@@ -410,12 +410,20 @@ class HipOps:
             if blocks is None:
                 seg_lens = meta.seg_lens if meta is not None and meta.seg_lens else \
                     self._segments(meta, token_segment, positions)[0]
-                flat, o = [], 0
-                for ln in seg_lens:
+                # (blocks with the most keys first: the compute units take them in order, and the last ones to start
+                # should be the short ones)
+                seg_starts = meta.seg_starts if meta is not None and meta.seg_starts else [0] * len(seg_lens)
+                keyed, o = [], 0
+                for ln, start in zip(seg_lens, seg_starts):
                     rows = ln * H
                     for t in range(0, rows, 64):
-                        flat += [o * H + t, min(64, rows - t)]
+                        nrows = min(64, rows - t)
+                        last = start + (t + nrows - 1) // H  # the position of the block's last token
+                        keys = last + 1 if not window else min(last + 1, window + -(-nrows // H))
+                        keyed.append((-keys, len(keyed), o * H + t, nrows))
                     o += ln
+                keyed.sort()
+                flat = [v for _, _, row0, nrows in keyed for v in (row0, nrows)]
                 blocks = torch.tensor(flat, dtype=torch.int32).to(q_lat.device)
                 if meta is not None:
                     meta.meta[key] = blocks
