@@ -66,6 +66,7 @@ class RequestEntry:
     serial: int = 0  # which life of which request this is: no two calls of add_request give the same
     freed_upto: list[int] = dataclasses.field(default_factory=list)  # per group: pages below this index (and beyond
     # the rule's kept prefix) have been given back
+    last_token: int = -1  # the last token that was committed (-1: none yet): what an embedding of token pairs needs
 
 
 @dataclasses.dataclass
@@ -298,10 +299,13 @@ class CacheManager:
                 table[j] = p
         e.reserved = n_new
 
-    def commit(self, rid) -> None:
+    def commit(self, rid, last_token: Optional[int] = None) -> None:
         """The step that wrote the reserved tokens is done: count them and give back
-        every page that no later query of this request can read."""
+        every page that no later query of this request can read.  ``last_token``: the last of the step's tokens
+        (kept as part of the request's state: the next step's first token has it as its neighbour)."""
         e = self.requests[rid]
+        if last_token is not None and e.reserved:
+            e.last_token = int(last_token)
         e.num_tokens += e.reserved
         e.reserved = 0
         e.steps += 1
@@ -358,6 +362,10 @@ class CacheManager:
 
     def slot(self, rid) -> int:
         return self.requests[rid].slot
+
+    def last_token(self, rid) -> int:
+        """The token before the request's next one (-1 at the start of the sequence)."""
+        return self.requests[rid].last_token
 
     def state_phase(self, rid) -> int:
         """Which half of its two-halved state the request's next step reads (it writes the other)."""

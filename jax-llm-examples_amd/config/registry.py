@@ -90,3 +90,4 @@ def _ensure_builtin() -> None:
     # importing the module registers the built-in architecture
     from ..parts import llama4 as _llama4  # noqa: F401
     from ..parts import rovidra as _rovidra  # noqa: F401
+    from ..parts import tiradra as _tiradra  # noqa: F401

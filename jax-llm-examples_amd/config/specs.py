@@ -58,12 +58,15 @@ class OrderEntry:
     ``layer`` indexes ``ModelPlan.layers``.  ``cache`` names the cache this run
     uses (an integer id; runs with the same id see the same keys and values).
     ``writes_cache`` is False for a run that only reads a cache another run
-    fills (that run must come earlier in the order).
+    fills (that run must come earlier in the order).  ``enters_pass``: this run is
+    the first of pass number ``enters_pass`` of a looped stretch of layers; the plan's
+    ``loop`` part says what happens to the residual stream there (``None``: nothing).
     """
 
     layer: int
     cache: int
     writes_cache: bool = True
+    enters_pass: int | None = None
 
 
 @dataclasses.dataclass(frozen=True)
@@ -77,6 +80,8 @@ class ModelPlan:
     # the model's two ends; None: a plain token table and a plain linear head (tied if tie_word_embeddings)
     embedding: PartSpec | None = None
     head: PartSpec | None = None
+    # what is done to the residual stream where a run of the order ``enters_pass`` (see parts/loop.py); None: no loop
+    loop: PartSpec | None = None
 
     def __post_init__(self) -> None:
         seen_write: dict[int, int] = {}
@@ -92,6 +97,8 @@ class ModelPlan:
                 seen_write[e.cache] = pos
             elif e.cache not in seen_write:
                 raise ValueError(f"order[{pos}] reads cache {e.cache} before any run has written it")
+            if e.enters_pass is not None and self.loop is None:
+                raise ValueError(f"order[{pos}] enters pass {e.enters_pass}, but the plan has no loop part")
 
 
 def default_order(num_layers: int) -> tuple[OrderEntry, ...]:

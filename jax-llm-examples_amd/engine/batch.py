@@ -53,6 +53,7 @@ class StepContext:
     num_tokens: int
     num_segments: int
     token_ids: torch.Tensor  # int32 [N]
+    prev_token_ids: torch.Tensor  # int32 [N]: the token before each token in its sequence, -1 for a first token
     positions: torch.Tensor  # int32 [N]
     token_segment: torch.Tensor  # int32 [N]
     cu_seqlens: torch.Tensor  # int32 [R + 1]
@@ -84,7 +85,7 @@ class StepLayout:
     def __init__(self, num_tokens: int, num_segments: int, num_wanted: int, widths: Sequence[int]) -> None:
         N, R = num_tokens, num_segments
         self.num_tokens, self.num_segments, self.num_wanted, self.widths = N, R, num_wanted, list(widths)
-        fields = [("token_ids", N), ("positions", N), ("token_segment", N), ("cu_seqlens", R + 1),
+        fields = [("token_ids", N), ("prev_token_ids", N), ("positions", N), ("token_segment", N), ("cu_seqlens", R + 1),
                   ("context_lens", R), ("state_slots", R), ("state_phase", R), ("logits_indices", num_wanted)]
         for g, w in enumerate(self.widths):
             fields += [(f"block_table{g}", R * w), (f"slot_mapping{g}", N)]
@@ -115,7 +116,7 @@ def fill_step(layout: StepLayout, flat: np.ndarray, cache, entries: Sequence[Ste
     v = lambda name: layout.view(flat, name)
     tok, pos, seg, cu = v("token_ids"), v("positions"), v("token_segment"), v("cu_seqlens")
     ctx_lens, slots, want = v("context_lens"), v("state_slots"), v("logits_indices")
-    phase = v("state_phase")
+    phase, prev = v("state_phase"), v("prev_token_ids")
     tables = [v(f"block_table{g.index}") for g in cache.groups]
     maps = [v(f"slot_mapping{g.index}") for g in cache.groups]
     seg_lens, seg_starts = [], []
@@ -131,11 +132,14 @@ def fill_step(layout: StepLayout, flat: np.ndarray, cache, entries: Sequence[Ste
             if not 0 <= t < vocab_size:
                 raise ValueError(f"request {e.rid!r}: token id outside 0..{vocab_size - 1}")
             tok[o], pos[o], seg[o] = t, start, i
+            prev[o] = cache.last_token(e.rid)
         else:
             t = np.asarray(e.tokens, dtype=np.int64)
             if t.min() < 0 or t.max() >= vocab_size:
                 raise ValueError(f"request {e.rid!r}: token id outside 0..{vocab_size - 1}")
             tok[o: o + n] = t
+            prev[o] = cache.last_token(e.rid)
+            prev[o + 1: o + n] = t[:-1]
             pos[o: o + n] = np.arange(start, start + n)
             seg[o: o + n] = i
         for x in e.want:
@@ -190,7 +194,7 @@ def context_over(layout: StepLayout, flat: torch.Tensor, cache, ops, dtype, devi
                                    seg_lens=seg_lens, seg_starts=seg_starts, decode_bucket=bucket))
     return StepContext(
         ops=ops, dtype=dtype, device=torch.device(device), num_tokens=layout.num_tokens, num_segments=R,
-        token_ids=d("token_ids"), positions=d("positions"), token_segment=d("token_segment"),
+        token_ids=d("token_ids"), prev_token_ids=d("prev_token_ids"), positions=d("positions"), token_segment=d("token_segment"),
         cu_seqlens=d("cu_seqlens"), context_lens=d("context_lens"), state_slots=d("state_slots"),
         state_phase=d("state_phase"),
         logits_indices=d("logits_indices"), groups=groups, seg_lens=seg_lens, seg_starts=seg_starts,

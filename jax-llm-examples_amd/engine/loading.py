@@ -64,7 +64,7 @@ def load_model(model_dir, dtype="bfloat16", device="cuda:0") -> DecoderModel:
     model.allocate()
     load_weights(model, os.fspath(model_dir), arch.bindings(cfg, model.plan),
                  optional_prefixes=getattr(arch, "optional_prefixes", ()),
-                 ignored_prefixes=getattr(arch, "ignored_prefixes", ()))
+                 ignored_prefixes=getattr(arch, "ignored_prefixes", ()))  # (finalizes the model's parts)
     return model
 
 

@@ -84,7 +84,7 @@ class ModelRunner:
                 cache.free(rid)
             raise
         for e in entries:
-            cache.commit(e.rid)
+            cache.commit(e.rid, last_token=e.tokens[-1])
         self.steps_run += 1
         self.tokens_run += num_tokens
         return logits

@@ -42,6 +42,13 @@ class ReferenceOps:
     def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
         return table[token_ids.long()].float()
 
+    def embed_pair(self, token_ids, prev_token_ids, table, pair_table, buckets: int, mul_prev: int, mul_cur: int):
+        """``table[token] + pair_table[(prev * mul_prev + token * mul_cur) mod buckets]``, and row ``buckets`` of the
+        pair table where there is no token before (``prev < 0``); float32."""
+        tok, prev = token_ids.long(), prev_token_ids.long()
+        row = torch.where(prev < 0, torch.full_like(tok, buckets), (prev * mul_prev + tok * mul_cur) % buckets)
+        return table[tok].float() + pair_table[row].float()
+
     # ------------------------------------------------------------------ norms
     def materialize(self, delta):
         """The tensor a branch output that is not formed yet stands for (float32)."""
@@ -51,7 +58,30 @@ class ReferenceOps:
             t = t * torch.sigmoid(g)
             t = t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + delta.eps)
             return t if delta.weight is None else t * delta.weight.float()
+        if hasattr(delta, "a"):  # a BranchSum
+            return delta.a.float() if delta.b is None else delta.a.float() + delta.b.float()
         return delta
+
+    def add_norm_pair(self, x, delta, injected, weight_a, weight_b, eps: float, out_dtype, second: bool = False,
+                      norm: bool = True):
+        """``x += delta`` (in place, float32; a tensor, a sum of two branches or ``None``), then with ``injected =
+        (rows, vector)`` ``x += rows`` (if any) and ``x += vector``; then ``h = x / sqrt(mean(x^2) + eps)`` once and
+        ``h * weight_a`` and (``second``) ``h * weight_b``, in the run dtype.  ``norm=False``: the sums only."""
+        if delta is not None:
+            x.add_(self.materialize(delta).float())
+        if injected is not None:
+            rows, vector = injected
+            if rows is not None:
+                x.add_(rows)
+            x.add_(vector.float())
+        if not norm:
+            return None, None
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        h_a = (h if weight_a is None else h * weight_a.float()).to(out_dtype)
+        h_b = None
+        if second:
+            h_b = (h if weight_b is None else h * weight_b.float()).to(out_dtype)
+        return h_a, h_b
 
     def add_norm_shift(self, x, delta, weight, eps: float, out_dtype, shift, ctx):
         """``x' = x + delta`` (a new tensor, float32; ``delta`` a tensor, a gated branch or ``None``), ``h =
@@ -103,13 +133,76 @@ class ReferenceOps:
         assert not tiled, "the plain ops read row-major weights"
         return h.float() @ w.float().t()
 
-    def swiglu_linear(self, h, w_gate_up):
-        return self.silu_mul(self.linear(h, w_gate_up))
+    def linear_bias(self, h, w, bias, bias_run=None):
+        """``h @ w.T + bias`` rounded once to the run dtype.  Returns ``(rows, bias still to be added or None)``:
+        a kernel set may leave the addition to the kernel that reads the rows next."""
+        out = h.float() @ w.float().t()
+        if bias is not None:
+            out = out + bias.float()
+        return out.to(h.dtype), None
 
-    def silu_mul(self, gate_up):
+    def swiglu_linear(self, h, w_gate_up, activation: str = "silu"):
+        return self.silu_mul(self.linear(h, w_gate_up), activation)
+
+    def silu_mul(self, gate_up, activation: str = "silu"):
+        """``act(gate) * up`` of the two halves of the last axis; ``act``: ``silu`` or ``gelu_tanh``."""
         f = gate_up.shape[-1] // 2
         g, u = gate_up[..., :f].float(), gate_up[..., f:].float()
-        return (torch.nn.functional.silu(g) * u).to(gate_up.dtype)
+        if activation == "gelu_tanh":
+            a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+        else:
+            a = torch.nn.functional.silu(g)
+        return (a * u).to(gate_up.dtype)
+
+    def sigmoid_mul(self, o, gate):
+        """``o * sigmoid(gate)`` element by element (``gate``: a view with the same shape), float32 inside."""
+        return (o.float() * torch.sigmoid(gate.float())).to(o.dtype)
+
+    def conv_qk_prepare(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
+                        value_dim: int, page_dim: int, prep, ctx, kv_cache, slot_mapping):
+        """From the projected rows ``[N, Hq*dk + Hk*dk + Hk*dv]`` to prepared queries and written pages.
+        ``u = proj + bias`` (rounded to the run dtype); every channel's causal convolution over time, ``y[t] =
+        sum_j conv_w[:, j] * u[t - taps + 1 + j]``, the rows before a segment's start from the request's state
+        (``state[slot, phase]``: ``[taps - 1, channels]``, the oldest first; zeros before the sequence's start) -
+        the last ``taps - 1`` rows of ``u`` go into ``state[slot, 1 - phase]``; ``y`` rounded to the run dtype; then
+        q and k turned by ``prep.rotation`` (sines and cosines times its magnitude) and divided by their root mean
+        square over the head; k and v written into their pages with heads of ``page_dim`` elements (zeros behind
+        the ``head_dim`` or ``value_dim`` real ones).  Returns q ``[N, Hq, page_dim]``."""
+        n = proj.shape[0]
+        dt = proj.dtype
+        hq, hk, dk, dv, D = num_heads, num_kv_heads, head_dim, value_dim, page_dim
+        u = proj.float() if bias is None else (proj.float() + bias.float())
+        u = u.to(dt).float()
+        y = u
+        if taps:
+            y = torch.zeros_like(u)
+            cu = ctx.cu_seqlens.tolist()
+            slots, phase = ctx.state_slots.tolist(), ctx.state_phase.tolist()
+            w = conv_w.float()
+            for s in range(len(cu) - 1):
+                lo, hi = cu[s], cu[s + 1]
+                rows = u[lo:hi]
+                if taps > 1:
+                    rows = torch.cat([state[slots[s], phase[s]].float(), rows], dim=0)  # [taps - 1 + len, C]
+                for j in range(taps):
+                    y[lo:hi] += w[:, j] * rows[j: j + hi - lo]
+                if taps > 1:
+                    state[slots[s], 1 - phase[s]] = rows[rows.shape[0] - (taps - 1):].to(state.dtype)
+            y = y.to(dt).float()
+        q = y[:, : hq * dk].reshape(n, hq, dk)
+        k = y[:, hq * dk: (hq + hk) * dk].reshape(n, hk, dk)
+        v = y[:, (hq + hk) * dk:].reshape(n, hk, dv)
+        q, k = self._turn(q, ctx.positions, prep.rotation), self._turn(k, ctx.positions, prep.rotation)
+        if prep.norm_eps is not None:
+            q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + prep.norm_eps)
+            k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + prep.norm_eps)
+        pad = lambda t: torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+        if kv_cache is not None:
+            ps = kv_cache.shape[3]
+            page, off = (slot_mapping // ps).long(), (slot_mapping % ps).long()
+            kv_cache[page, 0, :, off] = pad(k).to(kv_cache.dtype)
+            values_t(kv_cache)[page, :, :, off] = pad(v).to(kv_cache.dtype)
+        return pad(q).to(dt).contiguous()
 
     def batched_linear(self, a, w, tokens_first: bool = False):
         """``out[b] = a[b] @ w[b]`` for ``a [B, N, K]`` and ``w [B, K, M]`` (views with any strides);
@@ -133,7 +226,8 @@ class ReferenceOps:
             return x
         rd = int(rotation.rotary_dim) or x.shape[-1]
         ang = positions.float()[:, None] * rotation.inv_freq.float()[None, :]
-        sin, cos = torch.sin(ang), torch.cos(ang)
+        grow = float(getattr(rotation, "magnitude", 1.0))
+        sin, cos = torch.sin(ang) * grow, torch.cos(ang) * grow
         while sin.dim() < x.dim():
             sin, cos = sin.unsqueeze(1), cos.unsqueeze(1)
         head, rest = x[..., :rd], x[..., rd:]
@@ -149,7 +243,7 @@ class ReferenceOps:
     def latent_prepare(self, rows, num_heads: int, nope_dim: int, rope_dim: int, kv_rank: int, positions, rotation,
                        latent_norm, eps: float, latent_pages, rope_pages, slot_mapping, writes: bool,
                        latent_t_pages=None) -> None:
-        """``rows``: ``[N, H * (nope + rope) (+ kv_rank + rope)]``.  Turns the ``rope`` part of every head's
+        """``rows``: ``[N, H * (nope + rope) (+ kv_rank + rope) (+ anything else)]``.  Turns the ``rope`` part of every head's
         query in place; if the run writes its cache: RMS-norms the latent (the ``kv_rank`` numbers behind the
         queries) with ``latent_norm``, turns the shared key part (the last ``rope`` numbers) and writes both
         into their pages at ``slot = page * page_size + offset``."""
@@ -162,7 +256,7 @@ class ReferenceOps:
             c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps)
             if latent_norm is not None:
                 c = c * latent_norm.float()
-            kr = self._turn(rows[:, H * (dn + dr) + kv_rank:].float(), positions, rotation)
+            kr = self._turn(rows[:, H * (dn + dr) + kv_rank: H * (dn + dr) + kv_rank + dr].float(), positions, rotation)
             ps = latent_pages.shape[1]
             page, off = (slot_mapping // ps).long(), (slot_mapping % ps).long()
             latent_pages[page, off] = c.to(latent_pages.dtype)
@@ -171,11 +265,12 @@ class ReferenceOps:
                 latent_t_pages.view(latent_t_pages.shape[0], kv_rank, ps)[page, :, off] = c.to(latent_t_pages.dtype)
 
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
-                         token_segment, window, scale: float, meta=None, latent_t_pages=None):
+                         token_segment, window, scale: float, meta=None, latent_t_pages=None, sink=None):
         """For every token and head: softmax over the visible cached tokens ``j`` (``0 <= pos - j < window``;
         all earlier ones without a window) of ``(q_lat . c_j + q_r . k_j) * scale``, and the sum of the ``c_j``
         with those weights.  ``q_lat``: ``[H, N, kv_rank]``; ``q``: ``[N, H, nope + rope]`` whose rotated part is
-        ``q_r``.  Returns ``[N, H, kv_rank]``."""
+        ``q_r``.  ``sink``: float32 ``[H]``; ``exp(sink[h])`` is one more term of head ``h``'s denominator (no
+        key, no value, not scaled).  Returns ``[N, H, kv_rank]``."""
         H, n, r = q_lat.shape
         ps = latent_pages.shape[1]
         out = torch.empty(n, H, r, dtype=q_lat.dtype, device=q_lat.device)
@@ -190,7 +285,13 @@ class ReferenceOps:
             c = latent_pages[pages, off].float()  # [T, r]
             kr = rope_pages[pages, off].float()  # [T, rope]
             sc = (q_lat[:, i].float() @ c.t() + q[i, :, nope_dim:].float() @ kr.t()) * scale
-            out[i] = (torch.softmax(sc, dim=-1) @ c).to(out.dtype)
+            if sink is None:
+                pr = torch.softmax(sc, dim=-1)
+            else:
+                top = torch.maximum(sc.max(dim=-1, keepdim=True).values, sink.float()[:, None])
+                e = torch.exp(sc - top)
+                pr = e / (e.sum(dim=-1, keepdim=True) + torch.exp(sink.float()[:, None] - top))
+            out[i] = (pr @ c).to(out.dtype)
         return out
 
     # ------------------------------------------------------------------ attention
@@ -223,7 +324,8 @@ class ReferenceOps:
         if rot is not None:
             rd = int(rot.rotary_dim) or dh
             ang = positions.float()[:, None] * rot.inv_freq.float()[None, :]
-            sin, cos = torch.sin(ang)[:, None, :], torch.cos(ang)[:, None, :]
+            grow = float(getattr(rot, "magnitude", 1.0))
+            sin, cos = torch.sin(ang)[:, None, :] * grow, torch.cos(ang)[:, None, :] * grow
 
             def turn(x):
                 head, rest = x[..., :rd], x[..., rd:]

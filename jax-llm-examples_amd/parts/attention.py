@@ -4,7 +4,13 @@ One class covers both of Llama 4's attention layers, by parameters only:
 a position encoding that says how q and k are rotated (or none), an RMS norm of q
 and k or none (weightless after the rotation for Llama 4; weights and the place
 before the rotation are options), a retention rule (every earlier key, or the keys of the query's own chunk), and an
-optional position-dependent query scale.  Formulas:
+optional position-dependent query scale.  Further options, off for Llama 4: ``bias`` (q, k and v have
+biases, added in the projection), ``conv_taps`` (a short causal convolution over time on every channel of q, k and
+v, directly behind the projection: ``y[t] = sum_j w[:, j] * u[t - taps + 1 + j]``, zeros before the sequence's
+start; the last ``taps - 1`` projected rows of every request are its state, kept in two halves so that a step that
+is run twice reads what the first run read) and ``value_dim`` (values of another size than queries and keys: the
+pages then hold heads of the larger of the two sizes, rounded up to a multiple of 8, filled up with zeros, and
+the output projection skips the zeros).  Formulas:
 ``llama4/llama4_jax/model.py:891-955`` (projections, rotation, q/k norm, order of
 the cache write) and ``model.py:745-794`` (scores times ``softmax_scale``, causal
 mask, float32 softmax, values).
@@ -41,19 +47,51 @@ class Attention(Mixer):
         self.query_scale = None if qs is None else (float(qs.floor_scale), float(qs.attn_scale))
         self.prep = QKPreparation(norm_eps=self.qk_norm_eps, norm_first=self.qk_norm_first,
                                   query_scale=self.query_scale)
+        self.value_dim = int(spec.get("value_dim") or self.head_dim)
+        self.biased = bool(spec.get("bias", False))
+        self.conv_taps = int(spec.get("conv_taps") or 0)
+        # the path through the convolution kernel, which also rotates, norms, fills up and writes the pages
+        rot = self.position.rotation()
+        self.convolved = (self.conv_taps > 0 or self.value_dim != self.head_dim or self.biased
+                          or (rot is not None and rot.magnitude != 1.0))
+        if self.convolved and (self.qk_norm_weighted or self.qk_norm_first or self.query_scale is not None):
+            raise ValueError("the attention mixer's convolution path norms q and k without weights after the rotation "
+                             "and has no query scale")
+        # the head size of the pages
+        self.page_dim = self.head_dim if not self.convolved else -(-max(self.head_dim, self.value_dim) // 8) * 8
+        self.state_dtype = None
 
     def param_specs(self):
         hq, hk, dh, d = self.num_heads, self.num_kv_heads, self.head_dim, self.hidden
+        dv = self.value_dim
+        channels = (hq + hk) * dh + hk * dv
+        extra = {}
+        if self.biased:
+            extra["bqkv"] = ParamSpec((channels,), policy="float32", init=("normal", 0.3))
+        if self.conv_taps:
+            extra["conv"] = ParamSpec((channels, self.conv_taps), policy="float32", init=("normal", 0.6))
         return {
             # rows: q heads, then k heads, then v heads; each [out, in]
-            "wqkv": ParamSpec(((hq + 2 * hk) * dh, d)),
-            "wo": ParamSpec((d, hq * dh)),
+            "wqkv": ParamSpec((channels, d)),
+            "wo": ParamSpec((d, hq * dv)),
+            **extra,
             **({"q_norm": ParamSpec((dh,), policy="float32", init=("ones",)),
                 "k_norm": ParamSpec((dh,), policy="float32", init=("ones",))} if self.qk_norm_weighted else {}),
         }
 
+    @property
+    def channels(self) -> int:
+        return (self.num_heads + self.num_kv_heads) * self.head_dim + self.num_kv_heads * self.value_dim
+
+    def allocate(self, dtype, device) -> None:
+        super().allocate(dtype, device)
+        self.state_dtype = dtype
+
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(kv=(self.num_kv_heads, self.head_dim), retention=self.retention)
+        if self.conv_taps > 1:  # [half, tap, channel]: the last taps - 1 projected rows, as the projection left them
+            return CacheNeed(kv=(self.num_kv_heads, self.page_dim), retention=self.retention,
+                             state_shape=(2, self.conv_taps - 1, self.channels), state_dtype=self.state_dtype)
+        return CacheNeed(kv=(self.num_kv_heads, self.page_dim), retention=self.retention)
 
     graph_safe = True
 
@@ -64,14 +102,33 @@ class Attention(Mixer):
         self.prep.rotation = rot
         self.prep.norm_weight_q = self.params.get("q_norm")
         self.prep.norm_weight_k = self.params.get("k_norm")
+        self.bias_run = None
+        if self.biased:  # (the library's product adds a bias of its operands' dtype)
+            self.bias_run = self.params["bqkv"].to(self.params["wqkv"].dtype)
+        self.wo_padded = None
+        if self.page_dim != self.value_dim:  # the attention's output has page_dim elements a head: zeros' columns
+            wo = self.params["wo"]
+            padded = torch.zeros(wo.shape[0], self.num_heads, self.page_dim, dtype=wo.dtype, device=wo.device)
+            padded[:, :, : self.value_dim] = wo.view(wo.shape[0], self.num_heads, self.value_dim)
+            self.wo_padded = padded.view(wo.shape[0], self.num_heads * self.page_dim)
 
     def mixing_flops(self, start: int, count: int) -> float:
         """Two products (scores, values) over the keys each query can see."""
         keys = sum(p - first_needed_position(self.retention, p) + 1 for p in range(start, start + count))
-        return 4.0 * self.num_heads * self.head_dim * keys
+        return 2.0 * self.num_heads * (self.head_dim + self.value_dim) * keys
 
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
         ops = ctx.ops
+        if self.convolved:
+            # the projection (its bias added by the product where the library does it, else by the kernel below);
+            # then one kernel: convolution from the rows and the request's state, rotation, norm, pages
+            proj, bias = ops.linear_bias(h, self.params["wqkv"], self.params.get("bqkv"), self.bias_run)
+            q = ops.conv_qk_prepare(proj, bias, self.params.get("conv"), self.conv_taps, cache.state,
+                                    self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, self.page_dim,
+                                    self.prep, ctx, cache.kv if cache.writes else None, cache.slot_mapping)
+            o = ops.paged_attention(q, cache.kv, cache.block_table, ctx.positions, ctx.token_segment, self.retention,
+                                    self.softmax_scale, cache.attn_meta)
+            return ops.linear(o, self.params["wo"] if self.wo_padded is None else self.wo_padded)
         qkv = ops.linear(h, self.params["wqkv"])
         o = ops.attention_from_qkv(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx.positions, ctx.token_segment, self.prep,

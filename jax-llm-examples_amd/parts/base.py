@@ -231,11 +231,13 @@ class Rotation:
 
     ``inv_freq``: float32 ``[rotary_dim / 2]``; the angles are formed in float32 inside the kernel.
     ``pairing``: ``"adjacent"`` pairs ``(x[2j], x[2j+1])``; ``"half"`` pairs ``(x[j], x[j + rotary_dim/2])``.
-    ``rotary_dim``: the leading elements of a head that are rotated (the rest pass unchanged)."""
+    ``rotary_dim``: the leading elements of a head that are rotated (the rest pass unchanged).
+    ``magnitude``: a factor on every sine and cosine (the rotated elements grow by it)."""
 
     inv_freq: torch.Tensor
     pairing: str = "adjacent"
     rotary_dim: int = 0
+    magnitude: float = 1.0
 
 
 @dataclasses.dataclass
@@ -256,7 +258,8 @@ class QKPreparation:
     def plain(self) -> bool:
         """The case every kernel takes: adjacent pairs over the whole head, weightless norm after the rotation."""
         r = self.rotation
-        return ((r is None or (r.pairing == "adjacent" and r.rotary_dim in (0, 2 * r.inv_freq.numel())))
+        return ((r is None or (r.pairing == "adjacent" and r.rotary_dim in (0, 2 * r.inv_freq.numel())
+                               and r.magnitude == 1.0))
                 and self.norm_weight_q is None and self.norm_weight_k is None and not self.norm_first)
 
 

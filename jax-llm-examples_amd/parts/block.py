@@ -12,7 +12,7 @@ import torch
 
 from ..config.specs import LayerSpec
 from .base import ParamSpec, Part, build_feed_forward, build_mixer, build_norm
-from .residual import GatedBranch
+from .residual import BranchSum, GatedBranch
 
 _ARRANGEMENTS = {}
 
@@ -59,6 +59,41 @@ class PreNormBlock:
         else:
             h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input)
         residual.add(ff.forward(h, h32, ctx))
+
+
+@register_arrangement("parallel")
+class ParallelBlock:
+    """Both branches read the same stream, each through a norm of its own, and their outputs are added together::
+
+        x = x + (mixer(norm_a(x)) + feed_forward(norm_b(x)))
+
+    The two norms share their statistics (one kernel forms both rows); the sum of the two outputs stays pending on
+    the residual (a :class:`~.residual.BranchSum`).  The layer may have no feed-forward."""
+
+    def __init__(self, spec: LayerSpec) -> None:
+        self.spec = spec
+        self.mixer = build_mixer(spec.mixer)
+        self.mixer_norm = build_norm(spec.mixer_norm)
+        self.feed_forward = self.feed_forward_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+            if self.feed_forward_norm.eps != self.mixer_norm.eps:
+                raise ValueError("the two norms of a parallel layer share their statistics: one eps")
+
+    def parts(self):
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm}
+        if self.feed_forward is not None:
+            out.update(feed_forward=self.feed_forward, feed_forward_norm=self.feed_forward_norm)
+        return out
+
+    def forward(self, residual, ctx, cache) -> None:
+        ff = self.feed_forward
+        h_a, h_b = residual.normed_pair(ctx, self.mixer_norm.params.get("weight"),
+                                        None if ff is None else self.feed_forward_norm.params.get("weight"),
+                                        self.mixer_norm.eps)
+        y = self.mixer.forward(h_a, ctx, cache)
+        residual.add(BranchSum(y, None if ff is None else ff.forward(h_b, None, ctx)))
 
 
 class SigmoidGate(Part):

@@ -2,6 +2,9 @@
 
 ``token_embedding`` (``llama4/llama4_jax/model.py:1195``): row ``token`` of the table, as the first
 value of the float32 residual; optionally times a constant (``multiplier``).
+``token_pair_embedding``: the token's row plus a row of a second table chosen by a hash of (token before, token):
+``(prev * mul_prev + token * mul_cur) mod buckets``, and the table's extra last row for a sequence's first token.
+The token before is known to the step (``StepContext.prev_token_ids``; across steps the cache manager keeps it).
 ``linear_head`` (``model.py:1204``): float32 logits ``h @ W.T`` with a matrix of its own, or, with
 ``tied``, with the embedding's table; optionally plus a ``bias`` and squashed by a soft cap
 (``cap * tanh(logits / cap)``).  Llama 4 uses neither option: its ends are the two kernels alone.
@@ -34,6 +37,27 @@ class TokenEmbedding(Embedding):
         if self.multiplier is not None:
             x.mul_(self.multiplier)
         return x
+
+
+@register_embedding("token_pair_embedding")
+class TokenPairEmbedding(Embedding):
+    def __init__(self, spec) -> None:
+        super().__init__()
+        self.vocab_size, self.hidden = int(spec.vocab_size), int(spec.hidden_size)
+        self.buckets, self.mul_prev, self.mul_cur = int(spec.buckets), int(spec.mul_prev), int(spec.mul_cur)
+
+    graph_safe = True
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.vocab_size, self.hidden), init=("normal", 1.0)),
+                "pair": ParamSpec((self.buckets + 1, self.hidden), init=("normal", 0.5))}
+
+    def flops_per_token(self) -> float:
+        return 0.0
+
+    def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        return ctx.ops.embed_pair(token_ids, ctx.prev_token_ids, self.params["weight"], self.params["pair"],
+                                  self.buckets, self.mul_prev, self.mul_cur)
 
 
 @register_head("linear_head")

@@ -22,6 +22,9 @@ class DenseSwiGLU(FeedForward):
         super().__init__()
         self.hidden = int(spec.hidden_size)
         self.inter = int(spec.intermediate_size)
+        self.activation = str(spec.get("activation") or "silu")
+        if self.activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"unknown activation {self.activation!r} (silu, gelu_tanh)")
 
     def param_specs(self):
         return {
@@ -33,7 +36,10 @@ class DenseSwiGLU(FeedForward):
 
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
-        return ops.linear(ops.swiglu_linear(h, self.params["w_gate_up"]), self.params["w_down"])
+        if self.activation == "silu":
+            return ops.linear(ops.swiglu_linear(h, self.params["w_gate_up"]), self.params["w_down"])
+        return ops.linear(ops.swiglu_linear(h, self.params["w_gate_up"], activation=self.activation),
+                          self.params["w_down"])
 
 
 @register_feed_forward("moe_sigmoid_shared")

@@ -15,7 +15,10 @@ on how its request was cut into steps.
 Options as data: ``window`` (a query sees itself and the ``window - 1`` tokens before it; ``None``: all),
 ``retention`` (what the cache keeps: at least the window of every run that reads it), ``own_latent`` (False: the
 run projects no latent and reads a cache that another run writes), ``position`` (a rotary kind for ``q_r`` and
-``k_r``), ``latent_norm_eps``.
+``k_r``), ``latent_norm_eps``, ``sink`` (a learned number per head whose exponential is one more term of the
+softmax's denominator: it has no key and no value, is not scaled, and counts once) and ``output_gate`` (the heads'
+outputs are multiplied element by element with ``sigmoid(W_g h)`` before ``W_o``; ``W_g``'s rows ride behind the
+other projections' in ``w_in``).
 """
 from __future__ import annotations
 
@@ -44,6 +47,8 @@ class LatentAttention(Mixer):
         self.latent_norm_eps = float(spec.latent_norm_eps)
         self.position = build_position(spec.position, self.rope_dim)
         self.rotation = None
+        self.has_sink = bool(spec.get("sink", False))
+        self.output_gate = bool(spec.get("output_gate", False))
 
     @property
     def q_rows(self) -> int:
@@ -52,15 +57,19 @@ class LatentAttention(Mixer):
     def param_specs(self):
         h, d = self.num_heads, self.hidden
         kv = self.kv_rank + self.rope_dim if self.own_latent else 0
+        gate = h * self.value_dim if self.output_gate else 0
         specs = {
-            # rows: the heads' queries ([unrotated, rotated] per head), then the latent, then the shared rotated key
-            "w_in": ParamSpec((self.q_rows + kv, d), init=("normal", d ** -0.5)),
+            # rows: the heads' queries ([unrotated, rotated] per head), then the latent, then the shared rotated key,
+            # then the output gate's
+            "w_in": ParamSpec((self.q_rows + kv + gate, d), init=("normal", d ** -0.5)),
             "w_uk": ParamSpec((h * self.nope_dim, self.kv_rank), init=("normal", self.kv_rank ** -0.5)),
             "w_uv": ParamSpec((h * self.value_dim, self.kv_rank), init=("normal", self.kv_rank ** -0.5)),
             "wo": ParamSpec((d, h * self.value_dim), init=("normal", (h * self.value_dim) ** -0.5)),
         }
         if self.own_latent:
             specs["latent_norm"] = ParamSpec((self.kv_rank,), policy="float32", init=("uniform", 0.5, 1.5))
+        if self.has_sink:
+            specs["sink"] = ParamSpec((h,), policy="float32", init=("normal", 1.0))
         return specs
 
     def allocate(self, dtype, device) -> None:
@@ -98,6 +107,10 @@ class LatentAttention(Mixer):
     def flops_per_token(self) -> float:
         return 2.0 * (self.params["w_in"].numel() + self.params["wo"].numel())
 
+    @property
+    def gate_offset(self) -> int:
+        return self.q_rows + (self.kv_rank + self.rope_dim if self.own_latent else 0)
+
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
         ops = ctx.ops
         H, dn, dr, dv, r = self.num_heads, self.nope_dim, self.rope_dim, self.value_dim, self.kv_rank
@@ -115,7 +128,11 @@ class LatentAttention(Mixer):
         q_lat = ops.batched_linear(q[:, :, :dn].transpose(0, 1), self.params["w_uk"].view(H, dn, r))
         o_lat = ops.latent_attention(q_lat, q, dn, cache.pages["latent"], cache.pages["rope_key"], cache.block_table,
                                      ctx.positions, ctx.token_segment, self.window, self.softmax_scale,
-                                     cache.attn_meta, latent_t_pages=cache.pages.get("latent_t"))  # [N, H, r]
+                                     cache.attn_meta, latent_t_pages=cache.pages.get("latent_t"),
+                                     sink=self.params.get("sink"))  # [N, H, r]
         # the sums out of it: [H, N, r] x [H, r, dv], laid out [N, H * dv]
         o = ops.batched_linear(o_lat.transpose(0, 1), self.params["w_uv"].view(H, dv, r).transpose(1, 2), tokens_first=True)
-        return ops.linear(o.view(n, H * dv), self.params["wo"])
+        o = o.view(n, H * dv)
+        if self.output_gate:
+            o = ops.sigmoid_mul(o, rows[:, self.gate_offset: self.gate_offset + H * dv])
+        return ops.linear(o, self.params["wo"])

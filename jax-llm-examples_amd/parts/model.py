@@ -12,6 +12,7 @@ from ..config.specs import part
 from . import embedding as _ends  # noqa: F401  (registers the built-in embedding and head)
 from .base import CacheNeed, ParamSpec, Part, build_embedding, build_head, build_norm
 from .block import build_block
+from .loop import build_loop
 
 
 class DecoderModel:
@@ -23,6 +24,7 @@ class DecoderModel:
         self.embed = build_embedding(plan.embedding or part("token_embedding", vocab_size=plan.vocab_size,
                                                             hidden_size=plan.hidden_size))
         self.blocks = [build_block(spec) for spec in plan.layers]
+        self.loop = None if plan.loop is None else build_loop(plan.loop)
         self.final_norm = build_norm(plan.final_norm)
         self.lm_head = build_head(plan.head or part("linear_head", vocab_size=plan.vocab_size,
                                                     hidden_size=plan.hidden_size, tied=plan.tie_word_embeddings))
@@ -34,6 +36,8 @@ class DecoderModel:
         for i, b in enumerate(self.blocks):
             for name, p in b.parts().items():
                 out[f"layers.{i}.{name}"] = p
+        if self.loop is not None:
+            out["loop"] = self.loop
         out["final_norm"] = self.final_norm
         out["lm_head"] = self.lm_head
         return out
@@ -91,7 +95,12 @@ class DecoderModel:
         logits ``[len(ctx.logits_indices), vocab]``."""
         ops = ctx.ops
         residual = Residual(self.embed.forward(ctx.token_ids, ctx))
+        embedded = None
+        if self.loop is not None and getattr(self.loop, "needs_embedding_output", False):
+            embedded = residual.x.clone()  # (the stream itself is added to in place)
         for k, e in enumerate(self.plan.order):
+            if e.enters_pass is not None:
+                self.loop.enter(residual, embedded, e.enters_pass, ctx)
             gi = cache.group_of.get(e.cache)
             view = CacheView(cache_id=e.cache, writes=e.writes_cache, group=gi, state=cache.state.get(e.cache),
                              run_state=cache.run_state.get(k))

@@ -76,3 +76,40 @@ class RopeHalf(PositionEncoding):
         j = torch.arange(0, rd // 2, dtype=torch.float64)
         inv = torch.tensor(float(self.spec.theta), dtype=torch.float64) ** (-2.0 * j / rd)
         return Rotation(inv.to(torch.float32), pairing="half", rotary_dim=rd)
+
+
+def yarn_scaled_frequencies(inv_freq: torch.Tensor, base: float, dims: int, factor: float, original: float,
+                            fast: float, slow: float) -> torch.Tensor:
+    """Pairs that turn fewer than ``slow`` times over ``original`` positions are slowed by ``factor``, pairs that
+    turn more than ``fast`` times are kept, and between the two the mix goes linearly with the pair's index: the
+    pair that turns ``t`` times has the (fractional) index ``dims ln(original / (2 pi t)) / (2 ln base)``; the ramp
+    runs from the floor of that index for ``fast`` to its ceiling for ``slow`` (clipped to the pairs there are)."""
+    where = lambda turns: dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+    lo = max(math.floor(where(fast)), 0)
+    hi = min(math.ceil(where(slow)), dims - 1)
+    i = torch.arange(inv_freq.numel(), dtype=torch.float64)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return inv_freq / factor * ramp + inv_freq * (1.0 - ramp)
+
+
+@register_position("rope_yarn")
+class RopeYarn(PositionEncoding):
+    """Rotary embedding over adjacent pairs of the leading ``rotary_dim`` elements (default: all) with frequencies
+    ``theta ** (-2 j / rotary_dim)``, optionally stretched (``scaling = (factor, original, fast, slow)``, see
+    :func:`yarn_scaled_frequencies`); with a scaling the sines and cosines are also multiplied by
+    ``0.1 ln(factor) + 1`` (``Rotation.magnitude``)."""
+
+    def rotation(self) -> Rotation:
+        rd = int(self.spec.get("rotary_dim") or self.head_dim)
+        if rd % 2 or not 0 < rd <= self.head_dim:
+            raise ValueError(f"rotary_dim must be even and at most {self.head_dim}, got {rd}")
+        theta = float(self.spec.theta)
+        j = torch.arange(0, rd // 2, dtype=torch.float64)
+        inv = torch.tensor(theta, dtype=torch.float64) ** (-2.0 * j / rd)
+        magnitude = 1.0
+        scaling = self.spec.get("scaling")
+        if scaling:
+            factor, original, fast, slow = (float(v) for v in scaling)
+            inv = yarn_scaled_frequencies(inv, theta, rd, factor, original, fast, slow)
+            magnitude = 0.1 * math.log(factor) + 1.0
+        return Rotation(inv.to(torch.float32), pairing="adjacent", rotary_dim=rd, magnitude=magnitude)

@@ -21,12 +21,25 @@ class GatedBranch:
                            self.gate_bias, self.weight, self.eps)
 
 
+class BranchSum:
+    """The outputs of two branches that read the same rows (a layer with parallel branches): their sum
+    ``a + b``, formed in float32 by the kernel that adds it to the residual.  ``b`` may be ``None``."""
+
+    def __init__(self, a, b) -> None:
+        self.a, self.b = a, b
+        self.shape, self.dtype = a.shape, a.dtype
+
+    def rows(self, ops, idx) -> "BranchSum":
+        return BranchSum(ops.gather_rows(self.a, idx), None if self.b is None else ops.gather_rows(self.b, idx))
+
+
 class Residual:
     def __init__(self, x: torch.Tensor) -> None:
         assert x.dtype == torch.float32
         self._x = x
         self._deferred = None  # a norm (with its addition) that its consumer has been left to compute
         self.pending = None
+        self.injected = None  # (float32 rows or None, float32 vector): added after what is pending (see inject)
 
     @property
     def x(self) -> torch.Tensor:
@@ -41,9 +54,33 @@ class Residual:
             raise ValueError(f"branch output {tuple(delta.shape)} does not match residual {tuple(self.x.shape)}")
         self.pending = delta
 
+    def inject(self, rows, vector) -> None:
+        """``x + rows + vector`` (float32 ``[N, hidden]`` or ``None``, float32 ``[hidden]``), to be formed - after the
+        pending branch output is added - by the kernel that makes the next norm's rows."""
+        if self.injected is not None:
+            raise AssertionError("something is already to be injected into the residual")
+        self.injected = (rows, vector)
+
+    def _settle_injected(self, ctx) -> None:
+        """For consumers that do not know of injections: the sums are made now."""
+        if self.injected is not None:
+            x = self.value(ctx)
+            ctx.ops.add_norm_pair(x, None, self.injected, None, None, 0.0, ctx.dtype, norm=False)
+            self.injected = None
+
+    def normed_pair(self, ctx, weight_a, weight_b, eps: float):
+        """Adds what is pending and what is injected, and norms the rows once for two consumers: the same
+        statistics, each consumer's own weight (``weight_b`` ``None``: one consumer).  Returns ``(h_a, h_b or
+        None)`` in the run dtype."""
+        h_a, h_b = ctx.ops.add_norm_pair(self.x, self.pending, self.injected, weight_a, weight_b, eps, ctx.dtype,
+                                         second=weight_b is not None)
+        self.pending = self.injected = None
+        return h_a, h_b
+
     def normed(self, ctx, weight, eps: float, want32: bool = False, defer: bool = False):
         """``defer``: the part that takes the rows has said it accepts rows that are not computed yet (the
         kernel set's ``defer_norm``): it may then do addition and norm inside a launch of its own."""
+        self._settle_injected(ctx)
         if defer and hasattr(ctx.ops, "defer_norm"):
             p = ctx.ops.defer_norm(self.x, self.pending, weight, eps, ctx.dtype)
             self.pending, self._deferred = None, p
@@ -58,11 +95,13 @@ class Residual:
         ``[slots, 2, hidden]``, the last row of every request, one half read and the other written by a
         step).  The addition is not done in place: a row's kernel forms the row before it anew.  Returns
         ``(h, shifted h or None)`` in the run dtype."""
+        self._settle_injected(ctx)
         self._x, h, hs = ctx.ops.add_norm_shift(self.x, self.pending, weight, eps, ctx.dtype, shift, ctx)
         self.pending = None
         return h, hs
 
     def value(self, ctx) -> torch.Tensor:
+        """The stream with what is pending added (what is injected belongs to the next run and stays)."""
         if self.pending is not None:
             ctx.ops.add_residual(self.x, self.pending)
             self.pending = None
@@ -70,6 +109,7 @@ class Residual:
 
     def rows(self, ctx, idx: torch.Tensor) -> "Residual":
         """The residual of the chosen rows only (what is pending stays pending)."""
+        self._settle_injected(ctx)
         r = Residual(ctx.ops.gather_rows(self.x, idx))
         if self.pending is not None:
             if hasattr(self.pending, "rows"):
