@@ -1,0 +1,199 @@
+// Behind a fused q|k|v projection whose rows pass a short causal convolution over time before anything else:
+//     u[t]   = proj[t] + bias                                   (rounded to the run dtype: what the state keeps)
+//     y[t,c] = sum_j w[c, j] * u[t - taps + 1 + j, c]           (zeros before the sequence's start)
+// then, per head, the rotation of q and k (adjacent pairs of the leading rotary_dim elements, sines and cosines
+// times a magnitude), their division by the root mean square over the head, and the write of k and v into their
+// page.  Queries and keys have dk elements a head, values dv; the pages (and the queries handed on) hold heads of
+// D >= max(dk, dv) elements, the rest zeros, so that the attention kernels see one head size.
+//
+// The rows before a segment's first token come from the request's state: state[slot][half][taps - 1][C], the
+// oldest row first.  A step reads the half `phase` and writes the other, so a step that is run twice (once launch
+// by launch, once as a recorded graph) reads the same rows both times.
+//
+// One wavefront per (token, head); a lane holds elements lane, lane + 64, ... of the head, so the two elements of
+// a rotated pair lie in neighbouring lanes.  Everything in float32; the order of every sum depends on the sizes only.
+#include "common.h"
+
+using namespace jle;
+
+namespace {
+
+constexpr int kMaxPerLane = 8;  // heads of up to 512 elements
+
+template <typename PT, typename T>
+struct ConvArgs {
+  const PT* proj;      // [N, C]
+  const float* bias;   // [C] or null
+  const float* w;      // [C, taps] or null (taps == 0)
+  T* state;            // [slots, 2, taps - 1, C] or null (taps <= 1)
+  const int* token_segment;
+  const int* cu_seqlens;
+  const int* state_slots;
+  const int* state_phase;
+  const int* positions;
+  const int* slot_mapping;
+  const float* inv_freq;  // [rotary_dim / 2] or null
+  T* q_out;               // [N, Hq, D]
+  T* kv_cache;            // [pages, 2, Hkv, ps, D] (values [D][ps]) or null
+  float magnitude, norm_eps;  // norm_eps < 0: no norm
+  int taps, C, Hq, Hkv, dk, dv, D, ps, rotary_dim;
+};
+
+// the projected value of channel c in row `row`, with its bias, as the run dtype holds it
+template <typename PT, typename T>
+__device__ __forceinline__ float projected(const ConvArgs<PT, T>& a, size_t row, int c) {
+  float v = Num<PT>::load(a.proj + row * a.C + c);
+  if (a.bias != nullptr) v += a.bias[c];
+  return Num<T>::round(v);
+}
+
+template <typename PT, typename T>
+__global__ __launch_bounds__(64) void conv_qk_prepare_kernel(ConvArgs<PT, T> a) {
+  const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const bool is_q = h < a.Hq, is_v = h >= a.Hq + a.Hkv;
+  if (!is_q && a.kv_cache == nullptr) return;
+  const int dim = is_v ? a.dv : a.dk;
+  const int c0 = is_q ? h * a.dk : is_v ? (a.Hq + a.Hkv) * a.dk + (h - a.Hq - a.Hkv) * a.dv : h * a.dk;
+  const int seg = a.token_segment[n];
+  const int row0 = a.cu_seqlens[seg];
+  const int t = n - row0;  // the token's place in its segment
+  const int K = a.taps;
+  const T* old = nullptr;
+  if (K > 1) old = a.state + ((size_t)a.state_slots[seg] * 2 + a.state_phase[seg]) * (K - 1) * a.C;
+  float y[kMaxPerLane];
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int e = lane + 64 * i;
+    y[i] = 0.f;
+    if (e < dim) {
+      const int c = c0 + e;
+      if (K == 0) {
+        y[i] = projected(a, (size_t)n, c);
+      } else {
+        float acc = 0.f;
+        for (int j = 0; j < K; ++j) {
+          const int back = K - 1 - j;
+          const float u = t - back >= 0 ? projected(a, (size_t)(n - back), c)
+                                        : Num<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c);
+          acc = __builtin_fmaf(a.w[(size_t)c * K + j], u, acc);
+        }
+        y[i] = Num<T>::round(acc);
+      }
+    }
+  }
+  if (!is_v) {
+    const float pos = (float)a.positions[n];
+    const int rd = a.inv_freq != nullptr ? a.rotary_dim : 0;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int e = lane + 64 * i;
+      const float other = __shfl_xor(y[i], 1, 64);  // the pair's other element (every lane takes part)
+      if (e < rd) {
+        float sn, cs;
+        sincosf(pos * a.inv_freq[e >> 1], &sn, &cs);
+        sn *= a.magnitude;
+        cs *= a.magnitude;
+        y[i] = (e & 1) ? y[i] * cs + other * sn : y[i] * cs - other * sn;
+      }
+      ss = __builtin_fmaf(y[i], y[i], ss);
+    }
+    if (a.norm_eps >= 0.f) {
+      const float mul = 1.0f / sqrtf(wave_sum(ss) / (float)a.dk + a.norm_eps);
+#pragma unroll
+      for (int i = 0; i < kMaxPerLane; ++i) y[i] *= mul;
+    }
+  }
+  T* dst;
+  size_t stride = 1;
+  if (is_q) {
+    dst = a.q_out + ((size_t)n * a.Hq + h) * a.D;
+  } else {
+    const int slot = a.slot_mapping[n];
+    const int page = slot / a.ps, off = slot - page * a.ps;
+    const int hk = is_v ? h - a.Hq - a.Hkv : h - a.Hq;
+    T* plane = a.kv_cache + (((size_t)page * 2 + (is_v ? 1 : 0)) * a.Hkv + hk) * a.ps * a.D;
+    if (is_v) {
+      dst = plane + off;
+      stride = a.ps;
+    } else {
+      dst = plane + (size_t)off * a.D;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int e = lane + 64 * i;
+    if (e < a.D) Num<T>::store(dst + (size_t)e * stride, e < dim ? y[i] : 0.f);
+  }
+}
+
+// The state's other half: the last taps - 1 rows of u of every segment's request (older rows from the old half
+// where the segment is shorter than that).
+template <typename PT, typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(ConvArgs<PT, T> a) {
+  const int seg = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.C) return;
+  const int K = a.taps;
+  const int row0 = a.cu_seqlens[seg], len = a.cu_seqlens[seg + 1] - row0;
+  const size_t slot = (size_t)a.state_slots[seg];
+  const int phase = a.state_phase[seg];
+  const T* old = a.state + (slot * 2 + phase) * (K - 1) * a.C;
+  T* fresh = a.state + (slot * 2 + (1 - phase)) * (K - 1) * a.C;
+  for (int i = 0; i < K - 1; ++i) {
+    const int rel = len - (K - 1) + i;  // the row's place counted from the segment's first token
+    const float u = rel >= 0 ? projected(a, (size_t)(row0 + rel), c) : Num<T>::load(old + (size_t)(K - 1 + rel) * a.C + c);
+    Num<T>::store(fresh + (size_t)i * a.C + c, u);
+  }
+}
+
+template <typename PT, typename T>
+int launch_conv(const ConvArgs<PT, T>& a, int N, int R, hipStream_t s) {
+  hipLaunchKernelGGL((conv_qk_prepare_kernel<PT, T>), dim3(N, a.Hq + 2 * a.Hkv), dim3(64), 0, s, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  if (a.taps > 1) {
+    hipLaunchKernelGGL((conv_state_kernel<PT, T>), dim3(R, (a.C + 255) / 256), dim3(256), 0, s, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+  }
+  return 0;
+}
+
+}  // namespace
+
+// proj: [N, C] with C = (Hq + Hkv) * dk + Hkv * dv, float32 (proj_f32) or the run dtype (is_bf16).  N tokens in R
+// segments.  kv_cache null: this run writes no pages (the queries are prepared all the same).
+JLE_API int jle_conv_qk_prepare(const void* proj, int proj_f32, const float* bias, const float* conv_w, int taps,
+                                void* state, const int* token_segment, const int* cu_seqlens, const int* state_slots,
+                                const int* state_phase, const int* positions, const int* slot_mapping,
+                                const float* inv_freq, int rotary_dim, float magnitude, float norm_eps, void* q_out,
+                                void* kv_cache, int is_bf16, int N, int R, int Hq, int Hkv, int dk, int dv, int D,
+                                int ps, hipStream_t s) {
+  if (N <= 0) return 0;
+  if (Hq <= 0 || Hkv <= 0 || dk <= 0 || dv <= 0 || D < dk || D < dv || D > 64 * kMaxPerLane || taps < 0 || R <= 0 ||
+      Hq + 2 * Hkv > 65535 || R > 65535 * 16)
+    return JLE_BAD_ARG;
+  if ((taps > 0 && conv_w == nullptr) || (taps > 1 && (state == nullptr || state_slots == nullptr || state_phase == nullptr)))
+    return JLE_BAD_ARG;
+  if (inv_freq != nullptr && (rotary_dim <= 0 || rotary_dim % 2 || rotary_dim > dk)) return JLE_BAD_ARG;
+  if (kv_cache != nullptr && (slot_mapping == nullptr || ps <= 0)) return JLE_BAD_ARG;
+  if (!is_bf16 && !proj_f32) return JLE_BAD_ARG;
+  const int C = (Hq + Hkv) * dk + Hkv * dv;
+  if ((C + 255) / 256 > 65535) return JLE_BAD_ARG;
+#define JLE_CONV_ARGS(PT, T)                                                                                        \
+  ConvArgs<PT, T> a{(const PT*)proj, bias, conv_w, (T*)state, token_segment, cu_seqlens, state_slots, state_phase, \
+                    positions, slot_mapping, inv_freq, (T*)q_out, (T*)kv_cache, magnitude, norm_eps, taps, C, Hq,  \
+                    Hkv, dk, dv, D, ps, rotary_dim}
+  if (!is_bf16) {
+    JLE_CONV_ARGS(float, float);
+    return launch_conv(a, N, R, s);
+  }
+  if (proj_f32) {
+    JLE_CONV_ARGS(float, bf16_t);
+    return launch_conv(a, N, R, s);
+  }
+  JLE_CONV_ARGS(bf16_t, bf16_t);
+  return launch_conv(a, N, R, s);
+#undef JLE_CONV_ARGS
+}

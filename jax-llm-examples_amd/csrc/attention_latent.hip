@@ -3,7 +3,9 @@
 //     score_j = (q_lat . c_j + q_r . k_r_j) * scale      over the visible j (a window, or all earlier tokens)
 //     out     = sum_j softmax(score)_j c_j
 // where q_lat is the head's unrotated query taken into the latent's space by the caller and q_r its rotated part.
-// Float32 arithmetic on float32 or bfloat16 storage.
+// Float32 arithmetic on float32 or bfloat16 storage.  With a sink (one learned number per head) the softmax's
+// denominator has one more term, exp(sink): no key, no value, not scaled, counted once (where a query's keys are
+// shared between wavefronts: by the merge).
 //
 //   latent_prepare: rotates the q_r of every head in place, norms the latent, rotates the shared key part and
 //                   writes both into their pages (one block per token).
@@ -52,6 +54,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ rows, int ld, int H, int dn, int dr,
                                                              int R, const int* __restrict__ positions,
                                                              const float* __restrict__ inv_freq, int pairing, int rd,
+                                                             float magnitude /* on sines and cosines */,
                                                              const float* __restrict__ norm_w, float eps,
                                                              T* __restrict__ latent_pages, T* __restrict__ rope_pages,
                                                              T* __restrict__ latent_t_pages, int ps,
@@ -69,6 +72,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ row
     T* q = row + (size_t)h * (dn + dr) + dn;
     float sn, cs;
     sincosf(pos * inv_freq[j], &sn, &cs);
+    sn *= magnitude;
+    cs *= magnitude;
     const float u = Num<T>::load(q + ia), v = Num<T>::load(q + ib);
     Num<T>::store(q + ia, u * cs - v * sn);
     Num<T>::store(q + ib, v * cs + u * sn);
@@ -98,6 +103,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ row
     pair_index(pairing, rd, j, ia, ib);
     float sn, cs;
     sincosf(pos * inv_freq[j], &sn, &cs);
+    sn *= magnitude;
+    cs *= magnitude;
     const float u = Num<T>::load(kr + ia), v = Num<T>::load(kr + ib);
     Num<T>::store(rp + ia, u * cs - v * sn);
     Num<T>::store(rp + ib, v * cs + u * sn);
@@ -107,6 +114,16 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(T* __restrict__ row
 
 constexpr int kMaxAcc = 16;  // latent elements per lane: kv_rank up to 1024
 
+// What the sums over the keys (maximum m, denominator l) are multiplied with at the end: 1 / l, or with a sink
+// 1 / (l + exp(sink - m)), formed about the larger of m and the sink.
+__device__ __forceinline__ float closing_factor(float m, float l, const float* __restrict__ sink, int h) {
+  if (sink == nullptr) return 1.0f / l;
+  const float sk = sink[h];
+  const float top = fmaxf(m, sk);
+  const float a = expf(m - top);
+  return a / (l * a + expf(sk - top));
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void latent_attention_kernel(
     const T* __restrict__ q_lat /* [H, N, R] */, const T* __restrict__ q /* rows of q_ld: [H, dn + dr] first */,
@@ -114,7 +131,8 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     const T* __restrict__ latent_pages, const T* __restrict__ rope_pages, T* __restrict__ out /* [N, H, R] */,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, int window, float scale, int N, int H, int R, int ps, int splits, int tiles_per_split,
-    float* __restrict__ ws_ml, float* __restrict__ ws_o, int vec /* rows may be read 16 bytes at a time */) {
+    float* __restrict__ ws_ml, float* __restrict__ ws_o, int vec /* rows may be read 16 bytes at a time */,
+    const float* __restrict__ sink /* [H] or null */) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= N * H * splits) return;  // whole wavefront leaves; no block-wide barrier below
@@ -199,7 +217,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     }
     return;
   }
-  const float inv = bad ? __builtin_nanf("") : 1.0f / l;
+  const float inv = bad ? __builtin_nanf("") : closing_factor(m, l, sink, h);
   T* o = out + (size_t)nh * R;
 #pragma unroll
   for (int i = 0; i < kMaxAcc; ++i) {
@@ -212,7 +230,8 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ ws_ml,
                                                                      const float* __restrict__ ws_o,
-                                                                     T* __restrict__ out, int NH, int R, int splits) {
+                                                                     T* __restrict__ out, int NH, int R, int splits,
+                                                                     const float* __restrict__ sink, int H) {
   const int lane = threadIdx.x & 63;
   const int nh = blockIdx.x * 4 + wave_index();
   if (nh >= NH) return;
@@ -227,6 +246,11 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float
   bad = __any(bad);
   mx = wave_max(mx);
   float l = 0.f;
+  if (sink != nullptr) {  // (rows are token * H + head)
+    const float sk = sink[nh % H];
+    mx = fmaxf(mx, sk);
+    l = expf(sk - mx);
+  }
   float acc[kMaxAcc];
 #pragma unroll
   for (int i = 0; i < kMaxAcc; ++i) acc[i] = 0.f;
@@ -287,7 +311,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_segment,
     const int* __restrict__ block_table, int table_width, int window, float scale, const int* __restrict__ tiles,
     int num_tiles, int N, int H, int R, int ps, int splits, int steps_per_split, float* __restrict__ ws_ml,
-    float* __restrict__ ws_o) {
+    float* __restrict__ ws_o, const float* __restrict__ sink) {
   const int lane = threadIdx.x & 63, g = lane >> 4, r = lane & 15;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= num_tiles * splits) return;  // whole wavefront leaves; no block-wide barrier below
@@ -438,7 +462,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
       if (dt * 16 < R) *reinterpret_cast<f32x4*>(ws_o + slot * R + dt * 16 + g * 4) = acc[dt];
     return;
   }
-  const float inv = 1.0f / l;
+  const float inv = closing_factor(m, l, sink, h);
   bf16_t* o = out + (size_t)row * R;
 #pragma unroll
   for (int dt = 0; dt < NR * 2; ++dt) {
@@ -461,7 +485,7 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
     const bf16_t* __restrict__ latent, const bf16_t* __restrict__ latent_t, const bf16_t* __restrict__ rope,
     bf16_t* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_segment,
     const int* __restrict__ block_table, int table_width, int window, float scale, const int* __restrict__ blocks,
-    int N, int H, int R, int ps) {
+    int N, int H, int R, int ps, const float* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int drp = (dr + 31) & ~31;
   const int KS = R + drp + 8, VS = 40;  // row pitches in elements (16 bytes of padding: no bank conflicts)
@@ -667,7 +691,7 @@ __global__ __launch_bounds__(256) void latent_attention_lds_kernel(
     }
   }
   if (!row_ok) return;
-  const float inv = 1.0f / l;
+  const float inv = closing_factor(m, l, sink, h);
   bf16_t* o = out + (size_t)row * R;
 #pragma unroll
   for (int dt = 0; dt < NR * 2; ++dt) {
@@ -682,7 +706,7 @@ template <int NR>
 int launch_latent_lds(dim3 grid, size_t smem, hipStream_t s, const bf16_t* q_lat, const bf16_t* q, int q_ld, int dn,
                       int dr, const bf16_t* latent, const bf16_t* latent_t, const bf16_t* rope, bf16_t* out,
                       const int* positions, const int* token_segment, const int* block_table, int table_width,
-                      int window, float scale, const int* blocks, int N, int H, int R, int ps) {
+                      int window, float scale, const int* blocks, int N, int H, int R, int ps, const float* sink) {
   static size_t allowed = 0;  // (what this kernel has been given leave to use of the compute unit's shared memory)
   if (smem > allowed) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_lds_kernel<NR>),
@@ -692,7 +716,7 @@ int launch_latent_lds(dim3 grid, size_t smem, hipStream_t s, const bf16_t* q_lat
   }
   hipLaunchKernelGGL(latent_attention_lds_kernel<NR>, grid, dim3(256), smem, s, q_lat, q, q_ld, dn, dr, latent,
                      latent_t, rope, out, positions, token_segment, block_table, table_width, window, scale, blocks, N,
-                     H, R, ps);
+                     H, R, ps, sink);
   return 0;
 }
 
@@ -703,7 +727,8 @@ JLE_API int jle_latent_attention_lds(const void* q_lat, const void* q, int q_ld,
                                      const void* latent_pages, const void* latent_t_pages, const void* rope_pages,
                                      void* out, const int* positions, const int* token_segment,
                                      const int* block_table, int table_width, int window, float scale,
-                                     const int* blocks, int num_blocks, int N, int H, int R, int ps, hipStream_t s) {
+                                     const int* blocks, int num_blocks, int N, int H, int R, int ps,
+                                     const float* sink, hipStream_t s) {
   if (N <= 0 || num_blocks <= 0) return 0;
   if (!(R > 0 && R % 32 == 0 && R <= 512 && dr > 0 && dr % 8 == 0 && dr <= 64 && dn % 8 == 0 && q_ld % 8 == 0 &&
         ps % 8 == 0) ||
@@ -717,7 +742,7 @@ JLE_API int jle_latent_attention_lds(const void* q_lat, const void* q, int q_ld,
   rc = launch_latent_lds<NRV>(grid, smem, s, (const bf16_t*)q_lat, (const bf16_t*)q, q_ld, dn, dr,                 \
                               (const bf16_t*)latent_pages, (const bf16_t*)latent_t_pages, (const bf16_t*)rope_pages, \
                               (bf16_t*)out, positions, token_segment, block_table, table_width, window, scale, blocks, \
-                              N, H, R, ps)
+                              N, H, R, ps, sink)
   if (R <= 128)
     JLE_LATENT_LDS(4);
   else if (R <= 256)
@@ -743,7 +768,8 @@ JLE_API int jle_latent_attention_mfma(const void* q_lat, const void* q, int q_ld
                                       void* out, const int* positions, const int* token_segment,
                                       const int* block_table, int table_width, int window, float scale,
                                       const int* tiles, int num_tiles, int N, int H, int R, int ps, int splits,
-                                      int steps_per_split, float* ws_ml, float* ws_o, hipStream_t s) {
+                                      int steps_per_split, float* ws_ml, float* ws_o, const float* sink,
+                                      hipStream_t s) {
   if (N <= 0 || num_tiles <= 0) return 0;
   if (!jle_latent_attention_mfma_supported(R, dn, dr, q_ld, ps) || H <= 0 || window < 0 || tiles == nullptr ||
       latent_t_pages == nullptr || q_ld < H * (dn + dr))
@@ -756,7 +782,7 @@ JLE_API int jle_latent_attention_mfma(const void* q_lat, const void* q, int q_ld
   hipLaunchKernelGGL(latent_attention_mfma_kernel<NRV>, g, b, 0, s, (const bf16_t*)q_lat, (const bf16_t*)q, q_ld,   \
                      dn, dr, (const bf16_t*)latent_pages, (const bf16_t*)latent_t_pages, (const bf16_t*)rope_pages, \
                      (bf16_t*)out, positions, token_segment, block_table, table_width, window, scale, tiles,        \
-                     num_tiles, N, H, R, ps, splits, steps_per_split, ws_ml, ws_o)
+                     num_tiles, N, H, R, ps, splits, steps_per_split, ws_ml, ws_o, sink)
   if (R <= 128)
     JLE_LATENT_MFMA(4);
   else if (R <= 256)
@@ -767,7 +793,8 @@ JLE_API int jle_latent_attention_mfma(const void* q_lat, const void* q, int q_ld
   JLE_LAUNCH_CHECK();
   if (splits > 1) {
     dim3 gm((unsigned)(((long long)N * H + 3) / 4));
-    hipLaunchKernelGGL(latent_attention_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * H, R, splits);
+    hipLaunchKernelGGL(latent_attention_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * H, R, splits,
+                       sink, H);
     JLE_LAUNCH_CHECK();
   }
   return 0;
@@ -798,8 +825,8 @@ JLE_API int jle_swap_leading(const void* in, void* out, int A, int B, int row_by
 }
 
 JLE_API int jle_latent_prepare(void* rows, int ld, int H, int dn, int dr, int R, const int* positions,
-                               const float* inv_freq, int pairing, int rd, const float* norm_w, float eps,
-                               void* latent_pages, void* rope_pages, void* latent_t_pages, int ps,
+                               const float* inv_freq, int pairing, int rd, float magnitude, const float* norm_w,
+                               float eps, void* latent_pages, void* rope_pages, void* latent_t_pages, int ps,
                                const int* slot_mapping, int writes, int is_bf16, int N, hipStream_t s) {
   if (N <= 0) return 0;
   if (H <= 0 || dn < 0 || dr <= 0 || R <= 0 || rd % 2 || rd < 0 || rd > dr || (rd > 0 && inv_freq == nullptr))
@@ -809,11 +836,11 @@ JLE_API int jle_latent_prepare(void* rows, int ld, int H, int dn, int dr, int R,
     return JLE_BAD_ARG;
   if (is_bf16)
     hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, dim3(N), dim3(256), 0, s, (bf16_t*)rows, ld, H, dn, dr, R,
-                       positions, inv_freq, pairing, rd, norm_w, eps, (bf16_t*)latent_pages, (bf16_t*)rope_pages,
+                       positions, inv_freq, pairing, rd, magnitude, norm_w, eps, (bf16_t*)latent_pages, (bf16_t*)rope_pages,
                        (bf16_t*)latent_t_pages, ps, slot_mapping, writes);
   else
     hipLaunchKernelGGL(latent_prepare_kernel<float>, dim3(N), dim3(256), 0, s, (float*)rows, ld, H, dn, dr, R,
-                       positions, inv_freq, pairing, rd, norm_w, eps, (float*)latent_pages, (float*)rope_pages,
+                       positions, inv_freq, pairing, rd, magnitude, norm_w, eps, (float*)latent_pages, (float*)rope_pages,
                        (float*)latent_t_pages, ps, slot_mapping, writes);
   JLE_LAUNCH_CHECK();
   return 0;
@@ -825,7 +852,7 @@ JLE_API int jle_latent_attention(const void* q_lat, const void* q, int q_ld, int
                                  const void* rope_pages, void* out, const int* positions, const int* token_segment,
                                  const int* block_table, int table_width, int window, float scale, int is_bf16, int N,
                                  int H, int R, int ps, int splits, int tiles_per_split, float* ws_ml, float* ws_o,
-                                 hipStream_t s) {
+                                 const float* sink, hipStream_t s) {
   if (N <= 0) return 0;
   if (q_ld < H * (dn + dr) || H <= 0 || R <= 0 || R > 64 * kMaxAcc || dr <= 0 || dn < 0 || ps <= 0 || window < 0) return JLE_BAD_ARG;
   // rows are read 16 bytes at a time where every row starts at a multiple of 16 bytes
@@ -839,19 +866,21 @@ JLE_API int jle_latent_attention(const void* q_lat, const void* q, int q_ld, int
   if (is_bf16) {
     hipLaunchKernelGGL(latent_attention_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)q_lat, (const bf16_t*)q, q_ld, dn, dr,
                        (const bf16_t*)latent_pages, (const bf16_t*)rope_pages, (bf16_t*)out, positions, token_segment,
-                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o, vec);
+                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o, vec,
+                       sink);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(latent_attention_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * H, R,
-                         splits);
+                         splits, sink, H);
   } else {
     hipLaunchKernelGGL(latent_attention_kernel<float>, g, b, 0, s, (const float*)q_lat, (const float*)q, q_ld, dn, dr,
                        (const float*)latent_pages, (const float*)rope_pages, (float*)out, positions, token_segment,
-                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o, vec);
+                       block_table, table_width, window, scale, N, H, R, ps, splits, tiles_per_split, ws_ml, ws_o, vec,
+                       sink);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(latent_attention_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, N * H, R,
-                         splits);
+                         splits, sink, H);
   }
   JLE_LAUNCH_CHECK();
   return 0;

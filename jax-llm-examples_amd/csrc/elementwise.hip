@@ -24,6 +24,36 @@ JLE_API int jle_embed(const int* tok, const void* table, int is_bf16, float* out
   return 0;
 }
 
+// out = table[tok] + pair[(prev * mul_prev + tok * mul_cur) mod buckets], and row `buckets` of the pair table for a
+// token without a token before it (prev < 0); the hash in 64 bits.
+template <typename T>
+__global__ void embed_pair_kernel(const int* __restrict__ tok, const int* __restrict__ prev,
+                                  const T* __restrict__ table, const T* __restrict__ pair, float* __restrict__ out,
+                                  int D, int buckets, long long mul_prev, long long mul_cur) {
+  const size_t row = blockIdx.x;
+  const int t = tok[row], p = prev[row];
+  const long long r = p < 0 ? (long long)buckets : ((long long)p * mul_prev + (long long)t * mul_cur) % buckets;
+  const T* a = table + (size_t)t * D;
+  const T* b = pair + (size_t)r * D;
+  float* dst = out + row * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = Num<T>::load(a + d) + Num<T>::load(b + d);
+}
+
+JLE_API int jle_embed_pair(const int* tok, const int* prev, const void* table, const void* pair, int is_bf16,
+                           float* out, int N, int D, int buckets, long long mul_prev, long long mul_cur,
+                           hipStream_t s) {
+  if (N <= 0) return 0;
+  if (buckets <= 0 || mul_prev < 0 || mul_cur < 0) return JLE_BAD_ARG;
+  if (is_bf16)
+    hipLaunchKernelGGL(embed_pair_kernel<bf16_t>, dim3(N), dim3(256), 0, s, tok, prev, (const bf16_t*)table,
+                       (const bf16_t*)pair, out, D, buckets, mul_prev, mul_cur);
+  else
+    hipLaunchKernelGGL(embed_pair_kernel<float>, dim3(N), dim3(256), 0, s, tok, prev, (const float*)table,
+                       (const float*)pair, out, D, buckets, mul_prev, mul_cur);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------ add + rmsnorm
 // x (float32, the residual) += delta; out = x * rsqrt(mean(x^2) + eps) * weight.
 // delta is either a plain tensor or the sum of a token's expert outputs and the shared expert's:
@@ -244,20 +274,27 @@ JLE_API int jle_gather_rows(const void* src, const int* idx, void* out, int M, i
   return 0;
 }
 
-// ------------------------------------------------------------------ silu(gate) * up
-// in: [N, 2F] (gate columns, then up columns); out: [N, F]
-template <typename T>
+// ------------------------------------------------------------------ act(gate) * up
+// in: [N, 2F] (gate columns, then up columns); out: [N, F].  ACT 0: silu, z / (1 + exp(-z)); 1: the tanh form of
+// gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+template <int ACT>
+__device__ __forceinline__ float gate_act(float g) {
+  if (ACT == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.0f + expf(-g));
+}
+
+template <typename T, int ACT>
 __global__ void silu_mul_kernel(const T* __restrict__ in, T* __restrict__ out, int F) {
   const size_t row = blockIdx.y;
   const int f = blockIdx.x * blockDim.x + threadIdx.x;
   if (f >= F) return;
   const float g = Num<T>::load(in + row * 2 * F + f);
   const float u = Num<T>::load(in + row * 2 * F + F + f);
-  const float sg = g / (1.0f + expf(-g));
-  Num<T>::store(out + row * F + f, sg * u);
+  Num<T>::store(out + row * F + f, gate_act<ACT>(g) * u);
 }
 
 // bfloat16 rows whose halves are 16-byte aligned: 8 elements per thread
+template <int ACT>
 __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, int F) {
   const size_t row = blockIdx.y;
   const int f = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
@@ -270,23 +307,61 @@ __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ in, bf16_t* __
   for (int i = 0; i < 4; ++i) {
     const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
-    o[i] = pack_bf16(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+    o[i] = pack_bf16(gate_act<ACT>(g0) * u0, gate_act<ACT>(g1) * u1);
   }
   *reinterpret_cast<uint4*>(out + row * F + f) = uint4{o[0], o[1], o[2], o[3]};
 }
 
-JLE_API int jle_silu_mul(const void* in, void* out, int is_bf16, int N, int F, hipStream_t s) {
+template <int ACT>
+static int launch_act_mul(const void* in, void* out, int is_bf16, int N, int F, hipStream_t s) {
   if (N <= 0 || F <= 0) return 0;
   if (N > 65535 * 16) return JLE_BAD_ARG;
   dim3 g((F + 255) / 256, N), b(256);
   if (is_bf16 && F % 8 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
     dim3 g8((F / 8 + 255) / 256, N);
-    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, g8, b, 0, s, (const bf16_t*)in, (bf16_t*)out, F);
+    hipLaunchKernelGGL(silu_mul_bf16x8_kernel<ACT>, g8, b, 0, s, (const bf16_t*)in, (bf16_t*)out, F);
   } else if (is_bf16) {
-    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)in, (bf16_t*)out, F);
+    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, ACT>), g, b, 0, s, (const bf16_t*)in, (bf16_t*)out, F);
   } else {
-    hipLaunchKernelGGL(silu_mul_kernel<float>, g, b, 0, s, (const float*)in, (float*)out, F);
+    hipLaunchKernelGGL((silu_mul_kernel<float, ACT>), g, b, 0, s, (const float*)in, (float*)out, F);
   }
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+JLE_API int jle_silu_mul(const void* in, void* out, int is_bf16, int N, int F, hipStream_t s) {
+  return launch_act_mul<0>(in, out, is_bf16, N, F, s);
+}
+
+// act: 0 silu, 1 gelu (tanh form)
+JLE_API int jle_act_mul(const void* in, void* out, int is_bf16, int N, int F, int act, hipStream_t s) {
+  if (act == 0) return launch_act_mul<0>(in, out, is_bf16, N, F, s);
+  if (act == 1) return launch_act_mul<1>(in, out, is_bf16, N, F, s);
+  return JLE_BAD_ARG;
+}
+
+// out[n, c] = o[n, c] * sigmoid(gate[n * gate_ld + c]): the gate's rows are a slice of wider rows.
+template <typename T>
+__global__ void sigmoid_mul_kernel(const T* __restrict__ o, const T* __restrict__ gate, int gate_ld,
+                                   T* __restrict__ out, int C) {
+  const size_t row = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const float g = Num<T>::load(gate + row * gate_ld + c);
+  Num<T>::store(out + row * C + c, Num<T>::load(o + row * C + c) / (1.0f + expf(-g)));
+}
+
+JLE_API int jle_sigmoid_mul(const void* o, const void* gate, int gate_ld, void* out, int is_bf16, int N, int C,
+                            hipStream_t s) {
+  if (N <= 0 || C <= 0) return 0;
+  if (gate_ld < C || (C + 255) / 256 > 65535) return JLE_BAD_ARG;
+  dim3 g(N, (C + 255) / 256), b(256);
+  if (is_bf16)
+    hipLaunchKernelGGL(sigmoid_mul_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)o, (const bf16_t*)gate, gate_ld,
+                       (bf16_t*)out, C);
+  else
+    hipLaunchKernelGGL(sigmoid_mul_kernel<float>, g, b, 0, s, (const float*)o, (const float*)gate, gate_ld,
+                       (float*)out, C);
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -76,7 +76,7 @@ def main(argv=None) -> int:
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--page-size", type=int, default=16)
-    ap.add_argument("--max-requests", type=int, default=8, help="requests that may be live at once")
+    ap.add_argument("--max-requests", type=int, default=4, help="requests that may be live at once (state slots)")
     ap.add_argument("--poison", action="store_true",
                     help="fill the page pools with NaN, and every page again when it is given back: a page that is "
                          "read without having been written by its present holder then shows in the logits")

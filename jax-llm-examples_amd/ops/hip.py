@@ -60,14 +60,21 @@ _SIGNATURES = {
     "jle_add_norm_shift": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                            _vp, _i, _i, _i, _i, _vp],
     "jle_polynorm": [_vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
-    "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
+    "jle_latent_prepare": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _f, _vp, _f, _vp, _vp, _vp, _i, _vp, _i, _i, _i,
+                           _vp],
     "jle_swap_leading": [_vp, _vp, _i, _i, _i, _vp],
     "jle_latent_attention_lds": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
-                                 _i, _i, _vp],
+                                 _i, _i, _vp, _vp],
     "jle_latent_attention_mfma": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _i, _i, _i,
-                                  _i, _i, _i, _i, _vp, _vp, _vp],
+                                  _i, _i, _i, _i, _vp, _vp, _vp, _vp],
     "jle_latent_attention": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i,
-                             _vp, _vp, _vp],
+                             _vp, _vp, _vp, _vp],
+    "jle_embed_pair": [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _ll, _ll, _vp],
+    "jle_act_mul": [_vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_sigmoid_mul": [_vp, _vp, _i, _vp, _i, _i, _i, _vp],
+    "jle_add_norm_pair": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _vp],
+    "jle_conv_qk_prepare": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _f, _vp, _vp, _i, _i,
+                            _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -231,6 +238,49 @@ class HipOps:
         self._call("jle_embed", _p(token_ids), _p(table), self._is_bf16(table), _p(out), n, d)
         return out
 
+    def embed_pair(self, token_ids, prev_token_ids, table, pair_table, buckets: int, mul_prev: int, mul_cur: int):
+        """``table[token] + pair_table[(prev * mul_prev + token * mul_cur) mod buckets]`` (row ``buckets`` where
+        ``prev < 0``), float32."""
+        n, (v, d) = token_ids.numel(), table.shape
+        self._chk(token_ids, torch.int32, (n,), "token ids")
+        self._chk(prev_token_ids, torch.int32, (n,), "tokens before")
+        self._chk(table, None, (v, d), "embedding table")
+        self._chk(pair_table, table.dtype, (buckets + 1, d), "pair table")
+        out = torch.empty(n, d, dtype=torch.float32, device=table.device)
+        self._call("jle_embed_pair", _p(token_ids), _p(prev_token_ids), _p(table), _p(pair_table), self._is_bf16(table),
+                   _p(out), n, d, int(buckets), int(mul_prev), int(mul_cur))
+        return out
+
+    def add_norm_pair(self, x, delta, injected, weight_a, weight_b, eps: float, out_dtype, second: bool = False,
+                      norm: bool = True):
+        """``x += delta`` in place (``delta``: ``None``, a tensor, or a :class:`~..parts.residual.BranchSum` whose two
+        tensors the kernel adds up in float32), ``x += rows + vector`` for ``injected = (rows or None, vector)``,
+        then the row's statistics once and ``h * weight_a`` and (``second``) ``h * weight_b`` in the run dtype.
+        ``norm=False``: the sums only."""
+        n, d = x.shape
+        self._chk(x, torch.float32, (n, d), "residual")
+        a = b = None
+        if delta is not None:
+            delta = self.materialize(delta)
+            a, b = (delta.a, delta.b) if hasattr(delta, "a") else (delta, None)
+            self._chk(a, out_dtype, (n, d), "branch output")
+            if b is not None:
+                self._chk(b, out_dtype, (n, d), "second branch output")
+        rows = vec = None
+        if injected is not None:
+            rows, vec = injected
+            if rows is not None:
+                self._chk(rows, torch.float32, (n, d), "injected rows")
+            self._chk(vec, torch.float32, (d,), "injected vector")
+        for w in (weight_a, weight_b):
+            if w is not None:
+                self._chk(w, torch.float32, (d,), "norm weight")
+        h_a = torch.empty(n, d, dtype=out_dtype, device=x.device) if norm else None
+        h_b = torch.empty(n, d, dtype=out_dtype, device=x.device) if norm and second else None
+        self._call("jle_add_norm_pair", _p(x), _p(a), _p(b), _p(rows), _p(vec), _p(weight_a), _p(weight_b), float(eps),
+                   _p(h_a), _p(h_b), 1 if out_dtype == torch.bfloat16 else 0, n, d)
+        return h_a, h_b
+
     SHIFT_ROWS_PER_BLOCK = 4  # a block of the norm-and-shift kernel takes so many rows in a step of many tokens
     # (it forms the row before its first anew: with one row a block every row is formed twice)
 
@@ -311,6 +361,7 @@ class HipOps:
         self._chk(rows, None, None, "projected rows")
         self._chk(positions, torch.int32, (n,), "positions")
         pairing, rd, inv = 0, 0, None
+        magnitude = 1.0 if rotation is None else float(getattr(rotation, "magnitude", 1.0))
         if rotation is not None:
             rd = int(rotation.rotary_dim) or rope_dim
             pairing = {"adjacent": 0, "half": 1}[rotation.pairing]
@@ -325,7 +376,7 @@ class HipOps:
             if latent_norm is not None:
                 self._chk(latent_norm, torch.float32, (kv_rank,), "latent norm weight")
         self._call("jle_latent_prepare", _p(rows), ld, num_heads, nope_dim, rope_dim, kv_rank, _p(positions), _p(inv),
-                   pairing, rd, _p(latent_norm) if writes else None, float(eps),
+                   pairing, rd, magnitude, _p(latent_norm) if writes else None, float(eps),
                    _p(latent_pages) if writes else None, _p(rope_pages) if writes else None,
                    _p(latent_t_pages) if writes else None, latent_pages.shape[1] if writes else 0,
                    _p(slot_mapping) if writes else None, int(bool(writes)), self._is_bf16(rows), n)
@@ -338,7 +389,7 @@ class HipOps:
     LATENT_LDS_TILES = 1024  # from so many row tiles on: the kernel whose blocks share keys through shared memory
 
     def latent_attention(self, q_lat, q, nope_dim: int, latent_pages, rope_pages, block_table, positions,
-                         token_segment, window, scale: float, meta=None, latent_t_pages=None):
+                         token_segment, window, scale: float, meta=None, latent_t_pages=None, sink=None):
         """See ``attention_latent.hip``.  ``q_lat [H, N, kv_rank]``, ``q [N, H, nope + rope]`` (a view of the
         projected rows: the heads' queries lie at their start); returns ``[N, H, kv_rank]``.  In bfloat16, with the
         latent's transposed copy and sizes that fit, on the matrix cores; else in float32 arithmetic."""
@@ -355,12 +406,14 @@ class HipOps:
         self._chk(positions, torch.int32, (n,), "positions")
         self._chk(token_segment, torch.int32, (n,), "token segments")
         w = 0 if window is None else int(window)
+        if sink is not None:
+            self._chk(sink, torch.float32, (H,), "sinks")
         out = torch.empty(n, H, r, dtype=q_lat.dtype, device=q_lat.device)
         if (latent_t_pages is not None and q_lat.dtype == torch.bfloat16
                 and self._query("jle_latent_attention_mfma_supported", r, nope_dim, dr, q_ld, ps)):
             self._chk(latent_t_pages, latent_pages.dtype, (np_, ps, r), "transposed latent pages")
             return self._latent_attention_mfma(q_lat, q, q_ld, nope_dim, dr, latent_pages, latent_t_pages, rope_pages,
-                                               out, block_table, positions, token_segment, w, scale, meta)
+                                               out, block_table, positions, token_segment, w, scale, meta, sink)
         splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
         waves = n * H
         if waves < self.LATENT_SPLIT_BELOW:
@@ -380,11 +433,11 @@ class HipOps:
                 ws_o = torch.empty(waves * splits * r, dtype=torch.float32, device=q.device)
         self._call("jle_latent_attention", _p(q_lat), _p(q), q_ld, nope_dim, dr, _p(latent_pages), _p(rope_pages), _p(out),
                    _p(positions), _p(token_segment), _p(block_table), block_table.shape[1], w, float(scale),
-                   self._is_bf16(q_lat), n, H, r, ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
+                   self._is_bf16(q_lat), n, H, r, ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o), _p(sink))
         return out
 
     def _latent_attention_mfma(self, q_lat, q, q_ld, dn, dr, latent_pages, latent_t_pages, rope_pages, out,
-                               block_table, positions, token_segment, window, scale, meta):
+                               block_table, positions, token_segment, window, scale, meta, sink=None):
         H, n, r = q_lat.shape
         ps = latent_pages.shape[1]
         # row tiles: 16 consecutive (token, head) pairs of one segment
@@ -429,7 +482,8 @@ class HipOps:
                     meta.meta[key] = blocks
             self._call("jle_latent_attention_lds", _p(q_lat), _p(q), q_ld, dn, dr, _p(latent_pages),
                        _p(latent_t_pages), _p(rope_pages), _p(out), _p(positions), _p(token_segment), _p(block_table),
-                       block_table.shape[1], window, float(scale), _p(blocks), blocks.numel() // 2, n, H, r, ps)
+                       block_table.shape[1], window, float(scale), _p(blocks), blocks.numel() // 2, n, H, r, ps,
+                       _p(sink))
             return out
         splits, steps_per_split, ws_ml, ws_o = 1, 0, None, None
         if tiles < self.LATENT_MFMA_ITEMS:
@@ -450,10 +504,14 @@ class HipOps:
                 ws_o = torch.empty(n * H * splits * r, dtype=torch.float32, device=q_lat.device)
         self._call("jle_latent_attention_mfma", _p(q_lat), _p(q), q_ld, dn, dr, _p(latent_pages), _p(latent_t_pages),
                    _p(rope_pages), _p(out), _p(positions), _p(token_segment), _p(block_table), block_table.shape[1],
-                   window, float(scale), _p(plan), tiles, n, H, r, ps, splits, steps_per_split, _p(ws_ml), _p(ws_o))
+                   window, float(scale), _p(plan), tiles, n, H, r, ps, splits, steps_per_split, _p(ws_ml), _p(ws_o),
+                   _p(sink))
         return out
 
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
+        if hasattr(delta, "a"):  # the sum of two parallel branches: the kernel that knows it
+            h, _ = self.add_norm_pair(x, delta, None, weight, None, eps, out_dtype)
+            return h, (h.float() if want32 else None)
         if hasattr(delta, "gate"):  # a gated branch: the kernel that knows it (the sum goes into a new array)
             x_out, h, _ = self.add_norm_shift(x, delta, weight, eps, out_dtype, None, None)
             x.copy_(x_out)
@@ -485,7 +543,7 @@ class HipOps:
         return h.rows(want32) if isinstance(h, PendingNorm) else h
 
     def materialize(self, delta):
-        """The tensor an :class:`ExpertSum` stands for (float32)."""
+        """The tensor an :class:`ExpertSum` stands for (float32); anything else as it is."""
         if not isinstance(delta, ExpertSum):
             return delta
         n, d = delta.shape
@@ -495,6 +553,9 @@ class HipOps:
         return out
 
     def add_residual(self, x, delta) -> None:
+        if hasattr(delta, "a"):
+            self.add_norm_pair(x, delta, None, None, None, 0.0, delta.dtype, norm=False)
+            return
         if hasattr(delta, "gate"):
             x_out, _, _ = self.add_norm_shift(x, delta, None, 0.0, delta.y.dtype, None, None, do_norm=False)
             x.copy_(x_out)
@@ -525,12 +586,88 @@ class HipOps:
         out = torch.matmul(h, w.t())
         return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
 
-    def swiglu_linear(self, h, w_gate_up):
-        """``silu(h @ Wg.T) * (h @ Wu.T)`` with ``w_gate_up`` = gate rows, then up rows."""
+    def linear_bias(self, h, w, bias, bias_run=None):
+        """``h @ w.T + bias``.  Returns ``(rows, bias still to be added or None)``: the library's product adds the
+        bias itself (``bias_run``: the bias in the operands' dtype) and rounds once; the weight-streaming kernel
+        for few rows hands out float32 rows and leaves the bias to the kernel that reads them next."""
         h = self._rows(h)
+        if bias is None:
+            return self.linear(h, w), None
+        if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_LINEAR_ROWS and w.dtype == torch.bfloat16
+                and w.shape[1] % 8 == 0 and h.is_contiguous() and w.is_contiguous()):
+            return self.gemm_skinny(h, w, out_f32=True), bias
+        if bias_run is None:
+            bias_run = bias.to(h.dtype)
+        return torch.addmm(bias_run, h, w.t()), None
+
+    _ACTS = {"silu": 0, "gelu_tanh": 1}
+
+    def swiglu_linear(self, h, w_gate_up, activation: str = "silu"):
+        """``act(h @ Wg.T) * (h @ Wu.T)`` with ``w_gate_up`` = gate rows, then up rows; ``act``: ``silu`` or
+        ``gelu_tanh``."""
+        h = self._rows(h)
+        act = self._ACTS[activation]
         if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_DENSE_ROWS and h.shape[1] % 8 == 0:
-            return self.gemm_skinny(h, w_gate_up, swiglu=True)
-        return self.silu_mul(torch.matmul(h, w_gate_up.t()))
+            if act == 0:
+                return self.gemm_skinny(h, w_gate_up, swiglu=True)
+            return self.silu_mul(self.gemm_skinny(h, w_gate_up), activation)
+        return self.silu_mul(torch.matmul(h, w_gate_up.t()), activation)
+
+    def sigmoid_mul(self, o, gate):
+        """``o * sigmoid(gate)``; ``gate`` may be a slice of wider rows (its last axis contiguous)."""
+        n, c = o.shape
+        self._chk(o, None, (n, c), "rows")
+        if gate.dtype != o.dtype or tuple(gate.shape) != (n, c) or gate.stride(1) != 1 or not gate.is_cuda:
+            raise KernelError("the gate must have the rows' shape and dtype, its last axis contiguous")
+        out = torch.empty_like(o)
+        self._call("jle_sigmoid_mul", _p(o), _p(gate), gate.stride(0) if n > 1 else c, _p(out), self._is_bf16(o), n, c)
+        return out
+
+    def conv_qk_prepare(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
+                        value_dim: int, page_dim: int, prep, ctx, kv_cache, slot_mapping):
+        """See ``attention_conv.hip``: bias, causal convolution over time from the step's rows and the requests'
+        two-halved state, rotation and weightless norm of q and k, pages written with heads of ``page_dim``
+        elements.  Returns q ``[N, num_heads, page_dim]``."""
+        n = proj.shape[0]
+        hq, hk, dk, dv, D = num_heads, num_kv_heads, head_dim, value_dim, page_dim
+        channels = (hq + hk) * dk + hk * dv
+        dt = ctx.dtype
+        self._chk(proj, None, (n, channels), "projected rows")
+        if proj.dtype not in (dt, torch.float32):
+            raise KernelError(f"projected rows in {proj.dtype}, run dtype {dt}")
+        if prep.norm_weight_q is not None or prep.norm_weight_k is not None or prep.norm_first or prep.query_scale:
+            raise KernelError("the convolution path norms q and k without weights after the rotation, no query scale")
+        if bias is not None:
+            self._chk(bias, torch.float32, (channels,), "bias")
+        if taps:
+            self._chk(conv_w, torch.float32, (channels, taps), "convolution taps")
+        if taps > 1:
+            self._chk(state, dt, (state.shape[0], 2, taps - 1, channels), "convolution state")
+        rot = prep.rotation
+        inv_freq, rd, magnitude = None, 0, 1.0
+        if rot is not None:
+            if rot.pairing != "adjacent":
+                raise KernelError("the convolution path turns adjacent pairs")
+            rd = int(rot.rotary_dim) or dk
+            inv_freq, magnitude = self._chk(rot.inv_freq, torch.float32, (rd // 2,), "inv_freq"), float(rot.magnitude)
+        ps = 0
+        if kv_cache is not None:
+            ps = kv_cache.shape[3]
+            self._chk(kv_cache, dt, (kv_cache.shape[0], 2, hk, ps, D), "kv pages")
+            self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+        for t, what, shape in ((ctx.token_segment, "token segments", (n,)), (ctx.positions, "positions", (n,)),
+                               (ctx.cu_seqlens, "segment bounds", (ctx.num_segments + 1,)),
+                               (ctx.state_slots, "state slots", (ctx.num_segments,)),
+                               (ctx.state_phase, "state phases", (ctx.num_segments,))):
+            self._chk(t, torch.int32, shape, what)
+        q = torch.empty(n, hq, D, dtype=dt, device=proj.device)
+        self._call("jle_conv_qk_prepare", _p(proj), 1 if proj.dtype == torch.float32 else 0, _p(bias),
+                   _p(conv_w) if taps else None, int(taps), _p(state) if taps > 1 else None, _p(ctx.token_segment),
+                   _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(ctx.positions),
+                   _p(slot_mapping) if kv_cache is not None else None, _p(inv_freq), rd, magnitude,
+                   -1.0 if prep.norm_eps is None else float(prep.norm_eps), _p(q), _p(kv_cache),
+                   1 if dt == torch.bfloat16 else 0, n, ctx.num_segments, hq, hk, dk, dv, D, max(ps, 1))
+        return q
 
     def gemm(self, a, b, *, offsets=None, a_rows=None, scale=None, out_f32=False, rows=None):
         """The hand-written product ``C[r] = scale[r] * A[a_rows[r]] @ B[g(r)].T`` (see ``gemm_generic.hip``)."""
@@ -726,11 +863,14 @@ class HipOps:
             return self.gemm_grouped(h, w, out_f32=True, tiled=tiled)
         return self.gemm(h, w, out_f32=True)
 
-    def silu_mul(self, gate_up):
+    def silu_mul(self, gate_up, activation: str = "silu"):
         n, f2 = gate_up.shape
         self._chk(gate_up, None, None, "gate|up")
         out = torch.empty(n, f2 // 2, dtype=gate_up.dtype, device=gate_up.device)
-        self._call("jle_silu_mul", _p(gate_up), _p(out), self._is_bf16(gate_up), n, f2 // 2)
+        if activation == "silu":
+            self._call("jle_silu_mul", _p(gate_up), _p(out), self._is_bf16(gate_up), n, f2 // 2)
+        else:
+            self._call("jle_act_mul", _p(gate_up), _p(out), self._is_bf16(gate_up), n, f2 // 2, self._ACTS[activation])
         return out
 
     # ------------------------------------------------------------------ attention
@@ -747,6 +887,8 @@ class HipOps:
             if rot.pairing not in ("adjacent", "half"):
                 raise KernelError(f"rotary/norm kernel: unknown pairing {rot.pairing!r}")
             pairing = 0 if rot.pairing == "adjacent" else 1
+            if float(getattr(rot, "magnitude", 1.0)) != 1.0:
+                raise KernelError("rotary/norm kernel: sines and cosines with a magnitude go through conv_qk_prepare")
             if rd % 2 or not 0 < rd <= dh:
                 raise KernelError(f"rotary/norm kernel: {rd} rotated elements of a head of {dh}")
             self._chk(inv_freq, torch.float32, (rd // 2,), "inv_freq")
