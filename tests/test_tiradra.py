@@ -1,0 +1,600 @@
+"""The Tiradra decoder in the engine against the plain implementation (``plain_tiradra.py``): every mechanism
+alone; whole prompts, prefill against token-by-token decoding, portions down to two tokens, mixed batches with
+pages and state slots that are used again; keys far back and at page borders, in prompts and in decoding; the
+first tokens; long decoding; configurations whose sizes fit no fast path, are equal, 1 or absent; greedy
+generation through the engine's own entry point and scheduler; the configuration reader's errors.
+On the CPU with the plain ops (cache, state, batch and step logic), on the GPU with the HIP kernels."""
+import collections
+import json
+import math
+import os
+import subprocess
+import sys
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import plain_tiradra as P
+import traces
+from jax_llm_examples_amd import Engine, SamplingParams, load_model
+from jax_llm_examples_amd.cache import CacheManager, CacheView
+from jax_llm_examples_amd.config import ConfigError, get_architecture, load_config
+from jax_llm_examples_amd.config.specs import part
+from jax_llm_examples_amd.engine import StepEntry, build_context, get_ops
+from jax_llm_examples_amd.engine.replay import make_runner
+from jax_llm_examples_amd.parts.base import QKPreparation, build_position
+from jax_llm_examples_amd.parts.residual import BranchSum
+from jax_llm_examples_amd.weights import WeightsError
+from tiradra_configs import TIRADRA, TIRADRA_FAST, tiradra_config_json, write_tiradra
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEVICES = [pytest.param("cpu", id="cpu-plain-ops"), pytest.param("cuda:0", id="gpu-hip", marks=pytest.mark.gpu)]
+LENGTHS = {"TA": [1, 80, 33, 47, 64, 9, 130], "TB": [70, 2, 49, 96, 31, 17], "TC": [61, 3, 40, 90, 17],
+           "TD": [50, 1, 77, 18, 2], "TS": [161, 40, 5, 83], "TF": [420, 40, 170, 33], "TG": [150, 2, 61, 33, 97]}
+MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
+TOL = {"float32": 3e-5, "bfloat16": 4e-2}  # of the largest logit of the request
+# (bfloat16 with the sharp scores of TS: a rounding of a score of 20 by 2^-9 moves its weight by a twentieth)
+TOL_OF = {("TS", "bfloat16"): 1.5e-1}
+
+
+def _ops(device):
+    return get_ops(device, reference_ops=(device == "cpu"))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("tiradra")
+    return {name: write_tiradra(name, str(root / name), torch.float32) for name in TIRADRA}
+
+
+@pytest.fixture(scope="module")
+def folders_bf16(tmp_path_factory):
+    root = tmp_path_factory.mktemp("tiradra_bf16")
+    return {name: write_tiradra(name, str(root / name), torch.bfloat16) for name in {**TIRADRA, **TIRADRA_FAST}}
+
+
+def _step_ctx(device, seg_lens, seg_starts, slots, phases, dtype=torch.float32):
+    """The per-token and per-segment arrays a step's kernels read, made by hand."""
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    pos, seg, cu = [], [], [0]
+    for i, (n, s) in enumerate(zip(seg_lens, seg_starts)):
+        pos += list(range(s, s + n))
+        seg += [i] * n
+        cu.append(cu[-1] + n)
+    return types.SimpleNamespace(positions=i32(pos), token_segment=i32(seg), cu_seqlens=i32(cu), state_slots=i32(slots),
+                                 state_phase=i32(phases), dtype=dtype, num_segments=len(seg_lens))
+
+
+# ---------------------------------------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("device", DEVICES)
+def test_token_pair_embedding_alone(device):
+    """Rows of the pair table by the hash of (token before, token), in 64 bits; the extra row for a first token."""
+    g = torch.Generator().manual_seed(1)
+    V, D, buckets, a, b = 50000, 24, 1019, 3000000019, 1000003
+    table, pair = torch.randn(V, D, generator=g), torch.randn(buckets + 1, D, generator=g)
+    toks = [49999, 49998, 7, 0, 31337, 49999]
+    rows = P.bigram_rows(toks, buckets, a, b)
+    want = table[torch.tensor(toks)] + pair[torch.tensor(rows)]
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    got = _ops(device).embed_pair(i32(toks), i32([-1] + toks[:-1]), table.to(device), pair.to(device), buckets, a, b)
+    assert rows[0] == buckets and torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("width", [54, 64, 1000, 1536, 5000, 9000])
+def test_sum_of_two_branches_injection_and_two_norms_alone(device, width):
+    ops = _ops(device)
+    g = torch.Generator().manual_seed(width)
+    n, eps = 5, 1e-4
+    x, a, b, rows = (torch.randn(n, width, generator=g) for _ in range(4))
+    vec, w1, w2 = (torch.randn(width, generator=g) * 0.2 for _ in range(3))
+    dev = lambda t: t.to(device)
+    xs = x.double() + (a.double() + b.double()) + rows.double() + vec.double()
+    xd = dev(x.clone())
+    h1, h2 = ops.add_norm_pair(xd, BranchSum(dev(a), dev(b)), (dev(rows), dev(vec)), dev(1 + w1), dev(1 + w2), eps,
+                               torch.float32, second=True)
+    for got, want in ((xd, xs), (h1, P.centred_norm(xs, w1.double(), eps)), (h2, P.centred_norm(xs, w2.double(), eps))):
+        assert torch.allclose(got.cpu(), want.float(), rtol=2e-5, atol=3e-6), (got.cpu() - want.float()).abs().max()
+    # one branch, nothing injected, one norm; and the sums alone
+    xd = dev(x.clone())
+    h1, h2 = ops.add_norm_pair(xd, BranchSum(dev(a), None), None, dev(1 + w1), None, eps, torch.float32)
+    assert h2 is None and torch.allclose(h1.cpu(), P.centred_norm(x.double() + a.double(), w1.double(), eps).float(),
+                                         rtol=2e-5, atol=3e-6)
+    xd = dev(x.clone())
+    ops.add_norm_pair(xd, None, (None, dev(vec)), None, None, 0.0, torch.float32, norm=False)
+    assert torch.allclose(xd.cpu(), x + vec)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_gate_activation_and_sigmoid_gate_alone(device):
+    ops = _ops(device)
+    g = torch.Generator().manual_seed(2)
+    gu = torch.randn(6, 2 * 44, generator=g) * 3
+    want = P.gelu_tanh(gu[:, :44].double()) * gu[:, 44:].double()
+    got = ops.silu_mul(gu.to(device), "gelu_tanh").cpu()
+    assert torch.allclose(got, want.float(), rtol=2e-5, atol=2e-6)
+    o, wide = torch.randn(6, 20, generator=g), torch.randn(6, 50, generator=g)
+    got = ops.sigmoid_mul(o.to(device), wide.to(device)[:, 13:33]).cpu()
+    assert torch.allclose(got, (o.double() * torch.sigmoid(wide[:, 13:33].double())).float(), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("dims,scaling", [(8, (4.0, 64, 8.0, 2.0)), (32, (2.0, 4096, 32.0, 1.0)), (6, (2.5, 32, 6.0, 0.5)),
+                                           (2, (8.0, 16, 2.0, 1.0)), (64, (40.0, 100000, 3.0, 0.01)), (16, None)])
+def test_stretched_rotation_frequencies(dims, scaling):
+    """The position part's frequencies and magnitude against the plain formula: ramps that start before the first
+    pair, end behind the last, or have no width."""
+    top = None if scaling is None else dict(zip(("factor", "original", "fast", "slow"), scaling))
+    want, grow = P.rotary_frequencies(777.0, dims, top)
+    rot = build_position(part("rope_yarn", theta=777.0, rotary_dim=dims, scaling=scaling), dims + 4).rotation()
+    assert rot.pairing == "adjacent" and rot.rotary_dim == dims and rot.magnitude == pytest.approx(grow, rel=1e-12)
+    assert torch.allclose(rot.inv_freq.double(), torch.tensor(want, dtype=torch.float64), rtol=1e-6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("taps,dk,dv,rd", [(4, 16, 16, 16), (3, 16, 8, 8), (2, 8, 24, 4), (5, 6, 6, 6), (1, 10, 4, 4),
+                                            (0, 8, 8, 8), (4, 128, 64, 64)])
+def test_convolution_rotation_norm_and_pages_alone(device, taps, dk, dv, rd):
+    """Two sequences cut into unequal steps that share batches (portions shorter than the taps among them); the
+    state carries each sequence's last rows from step to step in the half that the step before wrote; a step run
+    twice before its commit gives the same twice."""
+    ops = _ops(device)
+    g = torch.Generator().manual_seed(taps * 100 + dk)
+    hq, hk, eps = 4, 2, 1e-5
+    D = -(-max(dk, dv) // 8) * 8
+    C = (hq + hk) * dk + hk * dv
+    lens = {"a": 23, "b": 9}
+    proj = {k: torch.randn(n, C, generator=g) for k, n in lens.items()}
+    bias, w = torch.randn(C, generator=g) * 0.3, torch.randn(C, max(taps, 1), generator=g) * 0.6
+    rot = build_position(part("rope_yarn", theta=300.0, rotary_dim=rd, scaling=(3.0, 32, 8.0, 1.0)), dk).rotation()
+    freqs, grow = P.rotary_frequencies(300.0, rd, {"factor": 3.0, "original": 32, "fast": 8.0, "slow": 1.0})
+    want = {}
+    for k, n in lens.items():
+        u = proj[k].double() + bias.double()
+        y = P.causal_conv(u, w.double()) if taps else u
+        q, kk, v = y[:, : hq * dk].view(n, hq, dk), y[:, hq * dk: (hq + hk) * dk].view(n, hk, dk), y[:, (hq + hk) * dk:].view(n, hk, dv)
+        pos = list(range(n))
+        want[k] = (P.unit_rms(P.rotate_adjacent(q, pos, freqs, grow), eps).float(),
+                   P.unit_rms(P.rotate_adjacent(kk, pos, freqs, grow), eps).float(), v.float())
+    dev = lambda t: t.to(device)
+    rot.inv_freq = dev(rot.inv_freq)
+    prep = QKPreparation(rotation=rot, norm_eps=eps)
+    ps, slot, pages_of = 4, {"a": 2, "b": 0}, {"a": list(range(0, 6)), "b": list(range(6, 9))}
+    kv = torch.full((9, 2, hk, ps, D), float("nan"), device=device)
+    state = torch.zeros(3, 2, max(taps - 1, 1), C, device=device) if taps > 1 else None
+    cuts = [[("a", 0, 5)], [("a", 5, 7), ("b", 0, 2)], [("b", 2, 9), ("a", 7, 8)], [("a", 8, 9)], [("a", 9, 23)]]
+    steps_done = {"a": 0, "b": 0}
+    got_q = {k: [] for k in lens}
+    for cut in cuts:
+        ctx = _step_ctx(device, [b - a for _, a, b in cut], [a for _, a, _ in cut], [slot[k] for k, _, _ in cut],
+                        [steps_done[k] & 1 for k, _, _ in cut])
+        rows = dev(torch.cat([proj[k][a:b] for k, a, b in cut]))
+        slots = torch.tensor([pages_of[k][t // ps] * ps + t % ps for k, a, b in cut for t in range(a, b)],
+                             dtype=torch.int32, device=device)
+        args = (rows, dev(bias), dev(w) if taps else None, taps, state, hq, hk, dk, dv, D, prep, ctx, kv, slots)
+        q1 = ops.conv_qk_prepare(*args).clone()
+        q2 = ops.conv_qk_prepare(*args)  # (again before the commit: the half it reads was not written)
+        assert torch.equal(q1, q2)
+        o = 0
+        for k, a, b in cut:
+            got_q[k].append(q1[o:o + b - a].cpu())
+            o += b - a
+            steps_done[k] += 1
+    for k, n in lens.items():
+        q = torch.cat(got_q[k])
+        assert torch.allclose(q[:, :, :dk], want[k][0], rtol=2e-4, atol=2e-5), (q[:, :, :dk] - want[k][0]).abs().max()
+        assert (q[:, :, dk:] == 0).all()
+        for t in range(n):
+            page, off = pages_of[k][t // ps], t % ps
+            key = kv[page, 0, :, off].cpu()
+            val = kv[page, 1].view(hk, D, ps)[:, :, off].cpu()
+            assert torch.allclose(key[:, :dk], want[k][1][t], rtol=2e-4, atol=2e-5) and (key[:, dk:] == 0).all()
+            assert torch.allclose(val[:, :dv], want[k][2][t], rtol=2e-4, atol=2e-5) and (val[:, dv:] == 0).all()
+
+
+def _mixer_alone(folder, device, layer, sizes, x, dtype="float32", page_size=16, sink=None):
+    """Runs one layer's mixer over the paged cache (and its per-request state) in the given portions."""
+    model = load_model(folder, dtype, device)
+    ops = _ops(device)
+    mixer = model.blocks[layer].mixer
+    if sink is not None:
+        mixer.params["sink"].fill_(sink)
+    pages = -(-sum(sizes) // page_size) + 1
+    cache = CacheManager({0: mixer.cache_need()}, page_size=page_size, num_pages=pages, max_requests=1, dtype=model.dtype,
+                         device=device, poison=True)
+    outs, o = [], 0
+    for n in sizes:
+        if not cache.has_request("r"):
+            cache.add_request("r")
+        cache.reserve("r", n)
+        ctx = build_context(ops, model.dtype, device, cache, [StepEntry("r", [0] * n, [])], model.config.vocab)
+        gctx = ctx.groups[0]
+        view = CacheView(0, True, kv=cache.groups[0].tensors.get(0), block_table=gctx.block_table,
+                         slot_mapping=gctx.slot_mapping, attn_meta=gctx, group=0, pages=cache.groups[0].pages[0],
+                         state=cache.state.get(0))
+        outs.append(mixer.forward(x[o:o + n].to(device).to(model.dtype), ctx, view).float().cpu())
+        cache.commit("r")
+        o += n
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layer", [("TA", 0), ("TA", 1), ("TA", 2), ("TA", 3), ("TB", 0), ("TB", 1), ("TB", 2),
+                                        ("TB", 3), ("TD", 1)])
+def test_mixers_alone(folders, device, name, layer):
+    """Each mixer over the paged cache, whole and in portions, equals the plain mixer (which forms every head's keys
+    and values, also from the latent): values of another size than keys, one kv head and as many as heads, partly
+    rotated heads, one to five taps and none, a sink, the output gate."""
+    plain = P.PlainTiradra(folders[name])
+    cfg, w = plain.cfg, plain.w
+    lc = cfg["layers"][layer]
+    T = 75
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(layer + 1))
+    want = P.MIXERS[lc["type"]](x.double(), lc["mixer"], w, f"l{layer}.mix.", list(range(T)), cfg["norm"]["eps"]).float()
+    for sizes in ([T], [30, 2, 17, 1, 1, 24]):
+        got = _mixer_alone(folders[name], device, layer, sizes, x)
+        assert torch.allclose(got, want, rtol=2e-4, atol=3e-5), (got - want).abs().max()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_the_sink_counts_once_whatever_the_keys_are_split_into(folders, device):
+    """A large sink takes most of every row's weight: the outputs shrink by what the plain softmax says, for a
+    query with one key and for one whose hundreds of keys are read by several wavefronts and merged; and the
+    output does change with the sink."""
+    name, layer = "TA", 1
+    plain = P.PlainTiradra(folders[name])
+    cfg = plain.cfg
+    lc = cfg["layers"][layer]
+    T = 300
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(4))
+    base = _mixer_alone(folders[name], device, layer, [T - 3, 1, 1, 1], x)
+    outs = {}
+    for sink in (3.0, -40.0):
+        plain.w[f"l{layer}.mix.sink"].fill_(sink)
+        want = P.latent_sink_attention(x.double(), lc["mixer"], plain.w, f"l{layer}.mix.", list(range(T)), cfg["norm"]["eps"]).float()
+        outs[sink] = _mixer_alone(folders[name], device, layer, [T - 3, 1, 1, 1], x, sink=sink)
+        assert torch.allclose(outs[sink], want, rtol=2e-4, atol=3e-5), (outs[sink] - want).abs().max()
+    assert (outs[3.0] - outs[-40.0]).abs().max() > 1e-2 and (base - outs[3.0]).abs().max() > 1e-3
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("decoding", [False, True])
+@pytest.mark.parametrize("special", [2, 15, 16, 255])
+def test_one_latent_key_that_stands_out_far_back(folders, device, decoding, special):
+    """One early token's shared key part is scaled up (the latent is normed, that part is not), so every later
+    query whose rotated part points its way puts all weight on it: at the start of the sequence, on a page's last
+    and first place, hundreds of tokens back; in a prompt and in decoding."""
+    name, layer = "TS", 1
+    plain = P.PlainTiradra(folders[name])
+    cfg, w = plain.cfg, plain.w
+    lc = cfg["layers"][layer]
+    T = 290
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(9))
+    x[special] *= 25.0
+    run = lambda rows: P.latent_sink_attention(rows.double(), lc["mixer"], w, f"l{layer}.mix.", list(range(T)),
+                                               cfg["norm"]["eps"]).float()
+    want = run(x)
+    sizes = [special + 3] + [1] * (T - special - 3) if decoding else [T]
+    got = _mixer_alone(folders[name], device, layer, sizes, x)
+    assert torch.allclose(got, want, rtol=3e-4, atol=3e-5), (got - want).abs().max()
+    x2 = x.clone()
+    x2[special] /= 25.0
+    assert (run(x2)[T - 1] - want[T - 1]).abs().max() > 1e-2  # (the last query does see it)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("decoding", [False, True])
+def test_sharp_attention_over_many_pages(folders, device, decoding):
+    """With scores this sharp a query's weight lies on one or two keys anywhere in the sequence: a key that is
+    missed or read from the wrong place, at a page's border or far back, moves the output by its whole size."""
+    name, layer = "TS", 0
+    plain = P.PlainTiradra(folders[name])
+    cfg, w = plain.cfg, plain.w
+    lc = cfg["layers"][layer]
+    T = 330
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(10))
+    want = P.conv_attention(x.double(), lc["mixer"], w, f"l{layer}.mix.", list(range(T)), cfg["norm"]["eps"]).float()
+    sizes = [T - 60] + [1] * 60 if decoding else [T]
+    got = _mixer_alone(folders[name], device, layer, sizes, x)
+    assert torch.allclose(got, want, rtol=3e-4, atol=3e-5), (got - want).abs().max()
+
+
+# ---------------------------------------------------------------------------------------------- whole models
+def _check(name, folder, dtype, device, mode, record=True, page_size=16, lengths=None):
+    lengths = lengths or (LENGTHS[name] + (LENGTHS[name][::-1] if mode == "mixed" else []))
+    reqs = traces.random_requests(tiradra_config_json(name)["vocab"], lengths, seed=5)
+    steps = MODES[mode](reqs)
+    runner = make_runner(folder, dtype, traces.max_live_tokens(steps), device, reference_ops=(device == "cpu"),
+                         poison=True, max_requests=4, page_size=page_size, decode_graphs=None if not record else False)
+    handed = [collections.Counter() for _ in runner.cache.groups]
+    for g, seen in zip(runner.cache.groups, handed):  # which pages every pool hands out, how often
+        def alloc(n, inner=g.pool.alloc, seen=seen):
+            pages = inner(n)
+            seen.update(pages)
+            return pages
+        g.pool.alloc = alloc
+    got = traces.run_trace(runner, steps)
+    if not record:
+        assert runner.graphs is not None and runner.graphs.replays > 0
+    if mode == "mixed":  # pages and slots were used again (a pool hands out the page that came back last)
+        assert all(max(seen.values()) > 1 for seen in handed)
+        assert len(reqs) > runner.cache.max_requests
+    runner.cache.check()
+    assert runner.cache.num_live() == 0 and all(g.pool.num_held == 0 for g in runner.cache.groups)
+    plain = P.PlainTiradra(folder)
+    for rid, toks in reqs.items():
+        ref = plain.logits(toks).float()
+        assert got[rid].shape == ref.shape and torch.isfinite(got[rid]).all(), f"{rid}: non-finite logits"
+        err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
+        bad = (err > TOL_OF.get((name, dtype), TOL[dtype])).nonzero().squeeze(-1).tolist()
+        assert not bad, f"{name} {dtype} {mode} {rid}: first wrong position {bad[0]} of {len(toks)}, error {err[bad[0]]:.3g}"
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(TIRADRA))
+def test_cpu_plain_ops_float32(folders, name, mode):
+    _check(name, folders[name], "float32", "cpu", mode)
+
+
+@pytest.mark.parametrize("page_size", [4, 64])
+def test_cpu_other_page_sizes(folders, page_size):
+    _check("TA", folders["TA"], "float32", "cpu", "mixed", page_size=page_size)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(TIRADRA))
+def test_gpu_float32(folders, name, mode):
+    _check(name, folders[name], "float32", "cuda:0", mode)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["tail", "mixed"])
+@pytest.mark.parametrize("name", list(TIRADRA))
+def test_gpu_float32_with_recorded_decode_steps(folders, name, mode):
+    _check(name, folders[name], "float32", "cuda:0", mode, record=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(TIRADRA) + list(TIRADRA_FAST))
+def test_gpu_bfloat16(folders_bf16, name, mode):
+    _check(name, folders_bf16[name], "bfloat16", "cuda:0", mode, record=(mode != "tail"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["TF", "TG"])
+def test_gpu_bfloat16_with_keys_shared_through_shared_memory(folders_bf16, monkeypatch, name, mode):
+    """Steps of many tokens go through the latent attention kernel whose blocks share their keys; here every step
+    of more than a few rows does."""
+    from jax_llm_examples_amd.ops.hip import HipOps
+
+    monkeypatch.setattr(HipOps, "LATENT_LDS_TILES", 2)
+    _check(name, folders_bf16[name], "bfloat16", "cuda:0", mode)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["TF", "TG"])
+def test_gpu_float32_at_vector_sizes(tmp_path, name):
+    folder = write_tiradra(name, str(tmp_path / name), torch.float32)
+    for mode in ("portions", "mixed"):
+        _check(name, folder, "float32", "cuda:0", mode)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", ["TA", "TC"])
+def test_residual_stream_behind_every_run_of_a_layer(folders, device, name):
+    """What a watcher of the step sees behind every run of a layer (a looped layer once per pass) equals the plain
+    model's stream: what a pass adds at its start belongs to the next run."""
+    folder = folders[name]
+    toks = traces.random_requests(128, [29], seed=2)["r0"]
+    want = []
+    P.PlainTiradra(folder).logits(toks, residuals=want)
+    runner = make_runner(folder, "float32", 64, device, reference_ops=(device == "cpu"), max_requests=2)
+    seen = []
+    runner.step([StepEntry("r", toks, [])], tap=lambda part, name, value: seen.append(value()) if name == "residual" else None)
+    assert len(seen) == len(want) == len(P.run_order(len(tiradra_config_json(name)["layers"]), tiradra_config_json(name)["loop"]))
+    for a, b in zip(seen, want):
+        assert torch.allclose(a.cpu(), b.float(), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_the_token_before_and_a_token_far_back_both_matter(folders, device):
+    """The logits at a step's first token change with the last token of the step before (the pair table's row) and
+    with a token 150 places back; the engine follows the plain model in both, in a prompt and in decoding."""
+    folder = folders["TS"]
+    plain = P.PlainTiradra(folder)
+    toks = traces.random_requests(128, [170], seed=4)["r0"]
+    i = 169
+
+    def logits_at(seq, decoding):
+        runner = make_runner(folder, "float32", 256, device, reference_ops=(device == "cpu"), max_requests=2)
+        if not decoding:
+            runner.step([StepEntry("r", seq[:i], [])])
+            return runner.step([StepEntry("r", seq[i:i + 1], [0])])[0].cpu().clone()
+        runner.step([StepEntry("r", seq[:140], [])])
+        for t in range(140, i):
+            runner.step([StepEntry("r", [seq[t]], [])])
+        return runner.step([StepEntry("r", [seq[i]], [0])])[0].cpu().clone()
+
+    for change in (i - 1, 19):
+        other = list(toks)
+        other[change] = (toks[change] + 1) % 128
+        for decoding in (False, True):
+            a, b = logits_at(toks, decoding), logits_at(other, decoding)
+            ra, rb = plain.logits(toks)[i].float(), plain.logits(other)[i].float()
+            assert (ra - rb).abs().max() > 1e-3, "the change does not show in the plain model: the test has no teeth"
+            assert torch.allclose(a, ra, atol=3e-4) and torch.allclose(b, rb, atol=3e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", ["TA", "TB"])
+def test_first_tokens_and_long_decoding(folders, device, name):
+    """A sequence fed one token at a time from its very first token, over many pages."""
+    folder = folders[name]
+    V = tiradra_config_json(name)["vocab"]
+    toks = traces.random_requests(V, [150], seed=6)["r0"]
+    runner = make_runner(folder, "float32", 192, device, reference_ops=(device == "cpu"), poison=True, max_requests=2)
+    rows = [runner.step([StepEntry("r", [t], [0])])[0].cpu().clone() for t in toks]
+    ref = P.PlainTiradra(folder).logits(toks).float()
+    err = (torch.stack(rows) - ref).abs().max(dim=-1).values / ref.abs().max()
+    assert float(err.max()) < TOL["float32"], f"first wrong position {int((err > TOL['float32']).nonzero()[0])}"
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_requests_in_a_batch_equal_each_alone(folders, device):
+    """The engine against itself: what a request gets beside others, in portions, on pages and slots that others
+    held before, is what it gets alone in one step."""
+    folder = folders["TA"]
+    reqs = traces.random_requests(300, [90, 7, 55, 31, 70, 12], seed=8)
+    run = lambda steps: traces.run_trace(make_runner(folder, "float32", traces.max_live_tokens(steps), device,
+                                                     reference_ops=(device == "cpu"), poison=True, max_requests=4), steps)
+    alone, together = run(traces.whole(reqs)), run(traces.mixed(reqs))
+    for rid in reqs:
+        assert torch.allclose(alone[rid], together[rid], rtol=1e-4, atol=2e-5), rid
+
+
+def _greedy(plain, prompt, n):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(plain.logits(seq)[-1].argmax()))
+    return seq[len(prompt):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", ["TA", "TB"])
+def test_greedy_generation_through_the_engine(folders, device, name):
+    """``Engine.generate``: the scheduler admits, cuts prompts into portions under a small token budget, decodes four
+    requests together, and frees; six requests on four slots."""
+    plain = P.PlainTiradra(folders[name])
+    V = plain.cfg["vocab"]
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (5, 61, 1, 33, 17, 2)]
+    eng = Engine(load_model(folders[name], "float32", device), reference_ops=(device == "cpu"), poison=True,
+                 cache_tokens=320, decode_batch_size=4, max_num_batched_tokens=48)
+    outs = eng.generate(prompts, SamplingParams(max_decode_length=12))
+    assert outs == [_greedy(plain, p, 12) for p in prompts]
+    eng.cache.check()
+    assert eng.cache.num_live() == 0 and all(g_.pool.num_held == 0 for g_ in eng.cache.groups)
+
+
+@pytest.mark.gpu
+def test_greedy_generation_in_bfloat16(folders_bf16):
+    """Every generated token is the plain model's first choice after the same tokens, or within bfloat16's
+    rounding of it."""
+    plain = P.PlainTiradra(folders_bf16["TF"])
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (40, 3, 120)]
+    eng = Engine(load_model(folders_bf16["TF"], "bfloat16", "cuda:0"), cache_tokens=1024, decode_batch_size=4,
+                 max_num_batched_tokens=64)
+    outs = eng.generate(prompts, SamplingParams(max_decode_length=16))
+    for p, out in zip(prompts, outs):
+        logits = plain.logits(list(p) + list(out)).float()
+        for i, tok in enumerate(out):
+            row = logits[len(p) + i - 1]
+            assert float(row.max() - row[tok]) <= 5e-2 * float(row.abs().max()), f"token {i} of {out}"
+
+
+@pytest.mark.gpu
+def test_command_line(folders, capsys):
+    """``python -m jax_llm_examples_amd.main`` picks the design by config.json like every other entry point."""
+    from jax_llm_examples_amd.main import main
+
+    plain = P.PlainTiradra(folders["TA"])
+    rc = main(["--ckpt-path", folders["TA"], "--dtype", "float32", "--prompt-ids", "5,6,7,8", "--prompt-ids", "9",
+               "--max-decode-length", "6", "--decode-batch-size", "2", "--max-seq-len", "64"])
+    assert rc == 0
+    lines = [json.loads(ln) for ln in capsys.readouterr().out.strip().splitlines()]
+    assert [ln["tokens"] for ln in lines] == [_greedy(plain, [5, 6, 7, 8], 6), _greedy(plain, [9], 6)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders_bf16, tmp_path, dtype):
+    """``bin/trace_run`` as a program, on a folder that holds config.json and bfloat16 weights."""
+    folder = folders_bf16["TA"]
+    reqs = traces.random_requests(300, [40, 9, 70, 21, 33], seed=11)
+    steps = traces.mixed(reqs)
+    out_dir = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out_dir), "--max-tokens", str(traces.max_live_tokens(steps))],
+                          input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [ln for ln in proc.stdout.splitlines() if ln.startswith("done")] == [f"done {s['step']}" for s in steps]
+    plain = P.PlainTiradra(folder)
+    ref = {rid: plain.logits(toks).float() for rid, toks in reqs.items()}
+    at = {rid: 0 for rid in reqs}
+    for s in steps:
+        got = np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(-1, 300)
+        o = 0
+        for e in s["entries"]:
+            for wnt in e["want"]:
+                r = ref[e["id"]][at[e["id"]] + wnt]
+                assert float((torch.from_numpy(got[o].copy()) - r).abs().max() / ref[e["id"]].abs().max()) < TOL[dtype]
+                o += 1
+            at[e["id"]] += len(e["tokens"])
+
+
+# ---------------------------------------------------------------------------------------------- configuration, weights
+def test_configuration_round_trip_and_plan(folders):
+    arch, cfg = load_config(folders["TA"])
+    assert arch is get_architecture("Tiradra")
+    assert arch.parse_config(json.loads(json.dumps(arch.config_to_dict(cfg)))) == cfg
+    plan = arch.plan(cfg)
+    # layers 1 and 2 three times in a row, every run with a cache of its own; a pass begins at layer 1
+    assert [(e.layer, e.cache, e.enters_pass) for e in plan.order] == [
+        (0, 0, None), (1, 1, 0), (2, 2, None), (1, 3, 1), (2, 4, None), (1, 5, 2), (2, 6, None), (3, 7, None)]
+    assert plan.layers[2].feed_forward is None and plan.layers[0].arrangement == "parallel"
+    assert plan.layers[0].mixer.value_dim == 8 and plan.layers[0].mixer.conv_taps == 3
+    model = load_model(folders["TA"], "float32", "cpu")
+    needs = model.cache_needs()
+    assert needs[0].kv == (2, 16) and needs[0].state_shape == (2, 2, 4 * 16 + 2 * 16 + 2 * 8)
+    assert needs[2].kv == (2, 24) and needs[2].state_shape == (2, 1, 2 * 8 + 2 * 8 + 2 * 24)
+    assert needs[1].paged[0] == ("latent", (32,)) and needs[1] == needs[3] == needs[5]
+    arch_b, cfg_b = load_config(folders["TB"])
+    plan_b = arch_b.plan(cfg_b)
+    assert plan_b.loop is None and plan_b.embedding.kind == "token_embedding" and plan_b.head.get("softcap") is None
+    assert all(e.enters_pass is None for e in plan_b.order)
+
+
+def test_configuration_errors():
+    arch = get_architecture("Tiradra")
+    good = tiradra_config_json("TA")
+
+    def broken(change):
+        top = json.loads(json.dumps(good))
+        change(top)
+        return top
+
+    for change, match in [
+        (lambda t: t["layers"][0]["mixer"].update(kv_heads=3), "no multiple"),
+        (lambda t: t["layers"][0]["mixer"].pop("scale"), "scale"),
+        (lambda t: t["layers"][0]["mixer"].update(window=4), "unknown key"),
+        (lambda t: t["layers"][0].update(type="convolution"), "not known"),
+        (lambda t: t["layers"][0]["mlp"].update(kind="experts"), "not known"),
+        (lambda t: t["layers"][0]["mixer"]["rot"].update(dims=3), "even"),
+        (lambda t: t["layers"][1]["mixer"]["rot"].update(dims=16), "at most"),
+        (lambda t: t["layers"][0]["mixer"]["rot"]["scaling"].pop("fast"), "fast"),
+        (lambda t: t["loop"].update(stop=9), "does not fit"),
+        (lambda t: t["embedding"]["bigram"].pop("buckets"), "buckets"),
+        (lambda t: t.pop("norm"), "norm"),
+    ]:
+        with pytest.raises(ConfigError, match=match):
+            arch.parse_config(broken(change))
+
+
+def test_weights_error_names_what_is_missing(folders, tmp_path):
+    from safetensors.torch import load_file, save_file
+
+    w = load_file(os.path.join(folders["TB"], "model.safetensors"))
+    w.pop("l0.mix.k.conv")
+    w["l2.mix.v.conv"] = torch.zeros(4, 3)  # that layer has no convolution
+    (tmp_path / "m").mkdir()
+    save_file(w, str(tmp_path / "m" / "model.safetensors"))
+    with open(os.path.join(folders["TB"], "config.json")) as f:
+        (tmp_path / "m" / "config.json").write_text(f.read())
+    with pytest.raises(WeightsError) as e:
+        load_model(str(tmp_path / "m"), "float32", "cpu")
+    assert e.value.missing == ["l0.mix.k.conv"] and e.value.unexpected == ["l2.mix.v.conv"]
