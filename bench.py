@@ -36,8 +36,10 @@ DESIGN_SIZES = {
 
 
 def design_configs(size: dict, layers: int):
-    """config.json of a Rovidra model (every second layer reads the latent of the layer before it) and of the
-    closest model the engine has: Llama 4 with dense layers only, rotary chunked attention, equal sizes."""
+    """config.json of a Rovidra model (every second layer reads the latent of the layer before it), of a Tiradra
+    model (every fourth layer attends over a latent, the others over convolved keys and values with 8 kv heads;
+    the inner layers run twice) and of the closest model the engine has: Llama 4 with dense layers only, rotary
+    chunked attention, equal sizes."""
     mixer = {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot"], "vdim": size["vdim"],
              "kv_rank": size["rank"], "scale": (size["dim"] + size["rot"]) ** -0.5,
              "rot": {"base": 500000.0, "dims": size["rot"]}, "mask": {"size": size["span"]}}
@@ -52,7 +54,19 @@ def design_configs(size: dict, layers: int):
              "rope_theta": 500000.0, "rope_scaling": None, "no_rope_layers": [1] * layers,
              "attention_chunk_size": size["span"], "use_qk_norm": True, "attn_temperature_tuning": False,
              "rms_norm_eps": 1e-5, "tie_word_embeddings": False}
-    return {"rovidra": rovidra, "llama4-dense": llama}
+    yarn = {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}
+    t_latent = {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot"], "vdim": size["vdim"],
+                "kv_rank": size["rank"], "scale": (size["dim"] + size["rot"]) ** -0.5,
+                "rot": {"base": 500000.0, "dims": size["rot"], "scaling": yarn}}
+    t_attn = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
+              "rot": {"base": 500000.0, "dims": 128, "scaling": yarn}}
+    tiradra = {"architecture": "Tiradra", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "logit_softcap": 30.0,
+               "layers": [{"type": "attention" if i % 4 else "latent_attention", "mixer": t_attn if i % 4 else t_latent,
+                           "mlp": {"kind": "dense", "ff": size["ff"]}} for i in range(layers)]}
+    if layers >= 3:
+        tiradra["loop"] = {"start": 1, "stop": layers - 1, "times": 2}
+    return {"rovidra": rovidra, "tiradra": tiradra, "llama4-dense": llama}
 
 
 def bench_designs(args) -> int:
@@ -74,6 +88,8 @@ def bench_designs(args) -> int:
     for size_name in names:
         size = DESIGN_SIZES[size_name]
         for design, top in design_configs(size, layers).items():
+            if args.design_names and design not in args.design_names.split(","):
+                continue
             arch = get_architecture(architecture_name(top))
             cfg = arch.parse_config(top)
             model = random_model(arch, cfg, seed=0, dtype=args.dtype, device=dev)
@@ -133,7 +149,7 @@ def bench_designs(args) -> int:
             out[f"{size_name}/{design}"] = res
             del runner, cache, model
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "prefill and decode tok/s of two designs at equal layer sizes, random weights",
+    print(json.dumps({"metric": "prefill and decode tok/s of the designs at equal layer sizes, random weights",
                       "dtype": dkey, "n_gpus": 1, "layers": layers, "sizes": {n: DESIGN_SIZES[n] for n in names},
                       "designs": out}), flush=True)
     return 0
@@ -159,8 +175,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--design-points", default="1@2048,8@2048,64@2048", help="decode steps of --designs: batch@context")
     ap.add_argument("--designs", default="", help="instead of the default workload: prefill and decode of the Rovidra "
-                    "design beside the dense Llama 4 layer of equal sizes, at the named sizes (comma-separated, of "
-                    + ", ".join(DESIGN_SIZES) + "; 'all')")
+                    "and Tiradra designs beside the dense Llama 4 layer of equal sizes, at the named sizes "
+                    "(comma-separated, of " + ", ".join(DESIGN_SIZES) + "; 'all')")
+    ap.add_argument("--design-names", default="", help="with --designs: only these of rovidra, tiradra, llama4-dense")
     args = ap.parse_args()
     if args.designs:
         return bench_designs(args)

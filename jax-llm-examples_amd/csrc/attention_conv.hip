@@ -1,6 +1,6 @@
 // Behind a fused q|k|v projection whose rows pass a short causal convolution over time before anything else:
 //     u[t]   = proj[t] + bias                                   (rounded to the run dtype: what the state keeps)
-//     y[t,c] = sum_j w[c, j] * u[t - taps + 1 + j, c]           (zeros before the sequence's start)
+//     y[t,c] = sum_j w[j, c] * u[t - taps + 1 + j, c]           (zeros before the sequence's start)
 // then, per head, the rotation of q and k (adjacent pairs of the leading rotary_dim elements, sines and cosines
 // times a magnitude), their division by the root mean square over the head, and the write of k and v into their
 // page.  Queries and keys have dk elements a head, values dv; the pages (and the queries handed on) hold heads of
@@ -24,7 +24,7 @@ template <typename PT, typename T>
 struct ConvArgs {
   const PT* proj;      // [N, C]
   const float* bias;   // [C] or null
-  const float* w;      // [C, taps] or null (taps == 0)
+  const float* w;      // [taps, C] (a tap's weights of all channels side by side) or null (taps == 0)
   T* state;            // [slots, 2, taps - 1, C] or null (taps <= 1)
   const int* token_segment;
   const int* cu_seqlens;
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64) void conv_qk_prepare_kernel(ConvArgs<PT, T> a) 
           const int back = K - 1 - j;
           const float u = t - back >= 0 ? projected(a, (size_t)(n - back), c)
                                         : Num<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c);
-          acc = __builtin_fmaf(a.w[(size_t)c * K + j], u, acc);
+          acc = __builtin_fmaf(a.w[(size_t)j * a.C + c], u, acc);
         }
         y[i] = Num<T>::round(acc);
       }
@@ -147,6 +147,154 @@ __global__ __launch_bounds__(256) void conv_state_kernel(ConvArgs<PT, T> a) {
   }
 }
 
+// The convolution alone, for sizes that the plain preparation kernels take afterwards: y[N, C] in the run dtype
+// (q heads, k heads, v heads as the projection laid them) and the state's other half, in one launch.  Blocks
+// 0 .. N - 1 of the grid's first axis take a token each, the R behind them a segment's state; a thread a channel.
+template <typename PT, typename T>
+__global__ __launch_bounds__(256) void conv_rows_kernel(ConvArgs<PT, T> a, T* __restrict__ y_out, int N) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.C) return;
+  const int K = a.taps;
+  if ((int)blockIdx.x >= N) {  // a segment's state
+    if (K <= 1) return;
+    const int seg = blockIdx.x - N;
+    const int row0 = a.cu_seqlens[seg], len = a.cu_seqlens[seg + 1] - row0;
+    const size_t slot = (size_t)a.state_slots[seg];
+    const int phase = a.state_phase[seg];
+    const T* old = a.state + (slot * 2 + phase) * (K - 1) * a.C;
+    T* fresh = a.state + (slot * 2 + (1 - phase)) * (K - 1) * a.C;
+    for (int i = 0; i < K - 1; ++i) {
+      const int rel = len - (K - 1) + i;
+      const float u = rel >= 0 ? projected(a, (size_t)(row0 + rel), c) : Num<T>::load(old + (size_t)(K - 1 + rel) * a.C + c);
+      Num<T>::store(fresh + (size_t)i * a.C + c, u);
+    }
+    return;
+  }
+  const int n = blockIdx.x;
+  float y;
+  if (K == 0) {
+    y = projected(a, (size_t)n, c);
+  } else {
+    const int seg = a.token_segment[n];
+    const int t = n - a.cu_seqlens[seg];
+    const T* old = nullptr;
+    if (K > 1) old = a.state + ((size_t)a.state_slots[seg] * 2 + a.state_phase[seg]) * (K - 1) * a.C;
+    float acc = 0.f;
+    for (int j = 0; j < K; ++j) {  // (the same sum, in the same order, as conv_qk_prepare_kernel's)
+      const int back = K - 1 - j;
+      const float u = t - back >= 0 ? projected(a, (size_t)(n - back), c)
+                                    : Num<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c);
+      acc = __builtin_fmaf(a.w[(size_t)j * a.C + c], u, acc);
+    }
+    y = Num<T>::round(acc);
+  }
+  Num<T>::store(y_out + (size_t)n * a.C + c, y);
+}
+
+// Eight neighbouring channels a thread (C a multiple of 8, every array 16-byte aligned): the same sums in the same
+// order as above, so which of the two kernels runs changes no bit.
+template <typename T>
+struct Row8;
+template <>
+struct Row8<float> {
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4*>(p + 4) = float4{v[4], v[5], v[6], v[7]};
+  }
+};
+template <>
+struct Row8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float* v) {
+    *reinterpret_cast<uint4*>(p) = uint4{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]),
+                                         pack_bf16(v[6], v[7])};
+  }
+};
+
+template <typename PT, typename T>
+__device__ __forceinline__ void projected8(const ConvArgs<PT, T>& a, size_t row, int c, const float* bias8, float* u) {
+  Row8<PT>::load(a.proj + row * a.C + c, u);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) u[i] = Num<T>::round(u[i] + bias8[i]);
+}
+
+template <typename PT, typename T>
+__global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T* __restrict__ y_out, int N) {
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= a.C) return;
+  const int K = a.taps;
+  float bias8[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) bias8[i] = 0.f;
+  if (a.bias != nullptr) Row8<float>::load(a.bias + c, bias8);
+  float u[8];
+  if ((int)blockIdx.x >= N) {  // a segment's state
+    if (K <= 1) return;
+    const int seg = blockIdx.x - N;
+    const int row0 = a.cu_seqlens[seg], len = a.cu_seqlens[seg + 1] - row0;
+    const size_t slot = (size_t)a.state_slots[seg];
+    const int phase = a.state_phase[seg];
+    const T* old = a.state + (slot * 2 + phase) * (K - 1) * a.C;
+    T* fresh = a.state + (slot * 2 + (1 - phase)) * (K - 1) * a.C;
+    for (int i = 0; i < K - 1; ++i) {
+      const int rel = len - (K - 1) + i;
+      if (rel >= 0) projected8(a, (size_t)(row0 + rel), c, bias8, u);
+      else Row8<T>::load(old + (size_t)(K - 1 + rel) * a.C + c, u);
+      Row8<T>::store(fresh + (size_t)i * a.C + c, u);
+    }
+    return;
+  }
+  const int n = blockIdx.x;
+  float y[8];
+  if (K == 0) {
+    projected8(a, (size_t)n, c, bias8, y);
+  } else {
+    const int seg = a.token_segment[n];
+    const int t = n - a.cu_seqlens[seg];
+    const T* old = nullptr;
+    if (K > 1) old = a.state + ((size_t)a.state_slots[seg] * 2 + a.state_phase[seg]) * (K - 1) * a.C;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = 0.f;
+    for (int j = 0; j < K; ++j) {
+      const int back = K - 1 - j;
+      if (t - back >= 0) projected8(a, (size_t)(n - back), c, bias8, u);
+      else Row8<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c, u);
+      float w8[8];
+      Row8<float>::load(a.w + (size_t)j * a.C + c, w8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = __builtin_fmaf(w8[i], u[i], y[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = Num<T>::round(y[i]);
+  }
+  Row8<T>::store(y_out + (size_t)n * a.C + c, y);
+}
+
+template <typename PT, typename T>
+int launch_conv_rows(const ConvArgs<PT, T>& a, void* y_out, int N, int R, hipStream_t s) {
+  const uintptr_t all = (uintptr_t)a.proj | (uintptr_t)a.bias | (uintptr_t)a.w | (uintptr_t)a.state | (uintptr_t)y_out;
+  if (a.C % 8 == 0 && all % 16 == 0)  // (by the sizes alone: the same kernel for every step of a model)
+    hipLaunchKernelGGL((conv_rows_vec_kernel<PT, T>), dim3(N + (a.taps > 1 ? R : 0), (a.C / 8 + 255) / 256), dim3(256),
+                       0, s, a, (T*)y_out, N);
+  else
+    hipLaunchKernelGGL((conv_rows_kernel<PT, T>), dim3(N + (a.taps > 1 ? R : 0), (a.C + 255) / 256), dim3(256), 0, s, a,
+                       (T*)y_out, N);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
 template <typename PT, typename T>
 int launch_conv(const ConvArgs<PT, T>& a, int N, int R, hipStream_t s) {
   hipLaunchKernelGGL((conv_qk_prepare_kernel<PT, T>), dim3(N, a.Hq + 2 * a.Hkv), dim3(64), 0, s, a);
@@ -196,4 +344,29 @@ JLE_API int jle_conv_qk_prepare(const void* proj, int proj_f32, const float* bia
   JLE_CONV_ARGS(bf16_t, bf16_t);
   return launch_conv(a, N, R, s);
 #undef JLE_CONV_ARGS
+}
+
+// The convolution alone: y [N, C] in the run dtype, C channels of any meaning; the state as above.
+JLE_API int jle_conv_rows(const void* proj, int proj_f32, const float* bias, const float* conv_w, int taps,
+                          void* state, const int* token_segment, const int* cu_seqlens, const int* state_slots,
+                          const int* state_phase, void* y_out, int is_bf16, int N, int R, int C, hipStream_t s) {
+  if (N <= 0) return 0;
+  if (C <= 0 || taps < 0 || R <= 0 || (C + 255) / 256 > 65535 || y_out == nullptr) return JLE_BAD_ARG;
+  if ((taps > 0 && conv_w == nullptr) || (taps > 1 && (state == nullptr || state_slots == nullptr || state_phase == nullptr)))
+    return JLE_BAD_ARG;
+  if (!is_bf16 && !proj_f32) return JLE_BAD_ARG;
+#define JLE_ROWS_ARGS(PT, T)                                                                                        \
+  ConvArgs<PT, T> a{(const PT*)proj, bias, conv_w, (T*)state, token_segment, cu_seqlens, state_slots, state_phase, \
+                    nullptr, nullptr, nullptr, nullptr, nullptr, 1.f, -1.f, taps, C, 0, 0, 0, 0, 0, 0, 0}
+  if (!is_bf16) {
+    JLE_ROWS_ARGS(float, float);
+    return launch_conv_rows(a, y_out, N, R, s);
+  }
+  if (proj_f32) {
+    JLE_ROWS_ARGS(float, bf16_t);
+    return launch_conv_rows(a, y_out, N, R, s);
+  }
+  JLE_ROWS_ARGS(bf16_t, bf16_t);
+  return launch_conv_rows(a, y_out, N, R, s);
+#undef JLE_ROWS_ARGS
 }

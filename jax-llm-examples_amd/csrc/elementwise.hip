@@ -340,6 +340,20 @@ JLE_API int jle_act_mul(const void* in, void* out, int is_bf16, int N, int F, in
   return JLE_BAD_ARG;
 }
 
+// x = cap * tanh(x / cap), in place
+__global__ void softcap_kernel(float* __restrict__ x, long long n, float cap) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
+JLE_API int jle_softcap(float* x, long long n, float cap, hipStream_t s) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f) || (n + 255) / 256 > 0x7fffffffll) return JLE_BAD_ARG;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, n, cap);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
 // out[n, c] = o[n, c] * sigmoid(gate[n * gate_ld + c]): the gate's rows are a slice of wider rows.
 template <typename T>
 __global__ void sigmoid_mul_kernel(const T* __restrict__ o, const T* __restrict__ gate, int gate_ld,

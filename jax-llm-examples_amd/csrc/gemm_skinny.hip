@@ -66,7 +66,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                           int tiled, const bf16_t* __restrict__ W_last,
                                                           int tiled_last, int num_groups, int slots,
                                                           int split_tiles, int split, float* __restrict__ ws,
-                                                          int* __restrict__ tickets) {
+                                                          int* __restrict__ tickets, int act) {
   static_assert(RT == 2 || !SWIGLU, "the fused activation needs the gate tile and the up tile");
   __shared__ float red[WAVES][RT * MT * 4][64];
   __shared__ __attribute__((aligned(16))) bf16_t turn[WAVES][RT * 16 * 72];  // (row-major weights only)
@@ -265,7 +265,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
       const int f = base + m;
       if (f < half) {
         const float gate = v0 * sc, up = v1 * sc;
-        store_out<OutT>(Y + (size_t)t * half + f, gate / (1.0f + expf(-gate)) * up);
+        // act 0: silu; 1: the tanh form of gelu
+        const float a = act == 1 ? 0.5f * gate * (1.0f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate)))
+                                 : gate / (1.0f + expf(-gate));
+        store_out<OutT>(Y + (size_t)t * half + f, a * up);
       }
     } else {
       const int c0 = base + m, c1 = base + 16 + m;
@@ -347,7 +350,7 @@ template <int MT, bool SW, typename OT>
 static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int variant, const void* X, const void* W,
                          void* Y, const int* offsets, const int* a_rows, const float* scale, int M, int Nout, int K,
                          int tiled, const void* W_last, int tiled_last, int zdim, int slots, int split_tiles,
-                         int split, float* ws, int* tickets) {
+                         int split, float* ws, int* tickets, int act) {
 #define LAUNCH(RT, WV, UN)                                                                                       \
   do {                                                                                                           \
     const int tiles_ = (xrows + 16 * (SW ? 1 : RT) - 1) / (16 * (SW ? 1 : RT));                                  \
@@ -356,7 +359,8 @@ static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int varian
     dim3 g(cut ? tiles_ + split_tiles * (split - 1) : tiles_, ytiles, zdim);                                     \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, SW, OT, WV, UN, (SW ? 2 : RT)>), g, dim3(WV * 64), 0, s,          \
                        (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K, tiled,    \
-                       (const bf16_t*)W_last, tiled_last, G, slots, cut ? split_tiles : 0, split, ws, tickets);  \
+                       (const bf16_t*)W_last, tiled_last, G, slots, cut ? split_tiles : 0, split, ws, tickets,   \
+                       act);                                                                                     \
     return 0;                                                                                                    \
   } while (0)
   switch (variant) {
@@ -416,12 +420,13 @@ JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* of
     variant = -variant;
   }
   const int zdim = slots > 0 ? slots : G;
+  const int act = swiglu == 2 ? 1 : 0;  // swiglu 1: silu(gate) * up; 2: gelu_tanh(gate) * up
   int rc;
 #define PICK(SW, OT)                                                                                             \
   do {                                                                                                           \
-    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last, zdim, slots, split_tiles, split, ws, tickets);      \
-    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last, zdim, slots, split_tiles, split, ws, tickets); \
-    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last, zdim, slots, split_tiles, split, ws, tickets);              \
+    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last, zdim, slots, split_tiles, split, ws, tickets, act);      \
+    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last, zdim, slots, split_tiles, split, ws, tickets, act); \
+    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last, zdim, slots, split_tiles, split, ws, tickets, act);              \
   } while (0)
   if (swiglu) {
     if (out_f32) PICK(true, float); else PICK(true, bf16_t);

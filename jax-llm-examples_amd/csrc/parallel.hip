@@ -7,6 +7,7 @@
 // One block per row, the row in registers (THREADS * EPT elements; wider rows are read again).  The sum of squares
 // is formed in an order that depends on the width only, so a token's rows do not depend on what else is in the step.
 #include "common.h"
+#include "rows.h"
 
 using namespace jle;
 
@@ -75,6 +76,68 @@ __global__ __launch_bounds__(THREADS) void add_norm_pair_kernel(PairArgs<DT> p) 
   }
 }
 
+// Rows whose width is a multiple of 4, all arrays 16-byte aligned: a thread takes CPT pieces of 4 neighbouring
+// elements (piece = thread, thread + THREADS, ...), every load of the row before its first store.
+template <typename DT, int THREADS, int CPT>
+__global__ __launch_bounds__(THREADS) void add_norm_pair_vec_kernel(PairArgs<DT> p) {
+  __shared__ float red[THREADS / 64];
+  const size_t base = (size_t)blockIdx.x * p.D;
+  const int D = p.D;
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f}, one = {1.f, 1.f, 1.f, 1.f};
+  f32x4_t v[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    v[i] = d < D ? load4<float>(p.x + base + d) : zero;
+  }
+  if (p.a != nullptr) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      if (d < D) {
+        f32x4_t t = load4<DT>(p.a + base + d);
+        if (p.b != nullptr) t += load4<DT>(p.b + base + d);
+        v[i] += t;
+      }
+    }
+  }
+  if (p.rows != nullptr) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      if (d < D) v[i] += load4<float>(p.rows + base + d);
+    }
+  }
+  if (p.vec != nullptr) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      if (d < D) v[i] += load4<float>(p.vec + d);
+    }
+  }
+  if (p.a != nullptr || p.rows != nullptr || p.vec != nullptr) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      if (d < D) store4<float>(p.x + base + d, v[i]);
+    }
+  }
+  if (p.h1 == nullptr) return;  // (the sums only)
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) ss = add_squares4(ss, v[i]);
+  const float inv = 1.0f / sqrtf(block_sum<THREADS>(ss, red) / (float)D + p.eps);
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    if (d < D) {
+      const f32x4_t h = v[i] * inv;
+      store4<DT>(p.h1 + base + d, p.w1 != nullptr ? h * load4<float>(p.w1 + d) : h * one);
+      if (p.h2 != nullptr) store4<DT>(p.h2 + base + d, p.w2 != nullptr ? h * load4<float>(p.w2 + d) : h * one);
+    }
+  }
+}
+
 // Rows wider than the registers hold: the sums are stored, the row read again for the statistics' use.
 template <typename DT, int THREADS>
 __global__ __launch_bounds__(THREADS) void add_norm_pair_wide_kernel(PairArgs<DT> p) {
@@ -99,6 +162,19 @@ __global__ __launch_bounds__(THREADS) void add_norm_pair_wide_kernel(PairArgs<DT
 template <typename DT>
 int launch_pair(const PairArgs<DT>& p, int N, hipStream_t s) {
   const int D = p.D;
+  // (which kernel: by the width and the arrays' alignment alone, never by the step's size)
+  const uintptr_t all = (uintptr_t)p.x | (uintptr_t)p.a | (uintptr_t)p.b | (uintptr_t)p.rows | (uintptr_t)p.vec |
+                        (uintptr_t)p.w1 | (uintptr_t)p.w2 | (uintptr_t)p.h1 | (uintptr_t)p.h2;
+  if (D % 4 == 0 && all % 16 == 0 && D >= 1024 && D <= 8192) {
+    if (D <= 2048)
+      hipLaunchKernelGGL((add_norm_pair_vec_kernel<DT, 256, 2>), dim3(N), dim3(256), 0, s, p);
+    else if (D <= 4096)
+      hipLaunchKernelGGL((add_norm_pair_vec_kernel<DT, 256, 4>), dim3(N), dim3(256), 0, s, p);
+    else
+      hipLaunchKernelGGL((add_norm_pair_vec_kernel<DT, 512, 4>), dim3(N), dim3(512), 0, s, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+  }
   if (D <= 256)
     hipLaunchKernelGGL((add_norm_pair_kernel<DT, 64, 4>), dim3(N), dim3(64), 0, s, p);
   else if (D <= 1024)

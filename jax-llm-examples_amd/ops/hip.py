@@ -71,8 +71,10 @@ _SIGNATURES = {
                              _vp, _vp, _vp, _vp],
     "jle_embed_pair": [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _ll, _ll, _vp],
     "jle_act_mul": [_vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_softcap": [_vp, _ll, _f, _vp],
     "jle_sigmoid_mul": [_vp, _vp, _i, _vp, _i, _i, _i, _vp],
     "jle_add_norm_pair": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _vp],
+    "jle_conv_rows": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_conv_qk_prepare": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _f, _vp, _vp, _i, _i,
                             _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -608,9 +610,7 @@ class HipOps:
         h = self._rows(h)
         act = self._ACTS[activation]
         if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_DENSE_ROWS and h.shape[1] % 8 == 0:
-            if act == 0:
-                return self.gemm_skinny(h, w_gate_up, swiglu=True)
-            return self.silu_mul(self.gemm_skinny(h, w_gate_up), activation)
+            return self.gemm_skinny(h, w_gate_up, swiglu=1 + act)  # (the activation in the product's epilogue)
         return self.silu_mul(torch.matmul(h, w_gate_up.t()), activation)
 
     def sigmoid_mul(self, o, gate):
@@ -622,6 +622,64 @@ class HipOps:
         out = torch.empty_like(o)
         self._call("jle_sigmoid_mul", _p(o), _p(gate), gate.stride(0) if n > 1 else c, _p(out), self._is_bf16(o), n, c)
         return out
+
+    def conv_attention(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
+                       value_dim: int, page_dim: int, prep, ctx, kv_cache, writes: bool, slot_mapping, block_table,
+                       retention, scale: float, meta=None):
+        """From the projected q|k|v rows to the attention output ``[N, num_heads * page_dim]``.  Where queries, keys
+        and values have one size and the rotation's magnitude can be told as a smaller eps of the norm behind it
+        (a rotation over the whole head turns nothing's length: ``m x / sqrt(m^2 s + eps) = x / sqrt(s + eps /
+        m^2)``), a kernel does bias, convolution and state, and the rows then go the way of any fused q|k|v rows
+        (:meth:`attention_from_qkv`: a step of single tokens is one more launch).  Everything else goes through
+        the kernel that also rotates, norms, fills heads up and writes the pages."""
+        rot = prep.rotation
+        rd = 0 if rot is None else (int(rot.rotary_dim) or head_dim)
+        m = 1.0 if rot is None else float(rot.magnitude)
+        if (head_dim == value_dim == page_dim and (m == 1.0 or (rd == head_dim and prep.norm_eps is not None))
+                and prep.norm_weight_q is None and prep.norm_weight_k is None and not prep.norm_first
+                and prep.query_scale is None):
+            rows = self.conv_rows(proj, bias, conv_w, taps, state, ctx)
+            plain = prep
+            if m != 1.0:
+                from ..parts.base import QKPreparation, Rotation
+
+                plain = getattr(prep, "_told_plainly", None)  # (made once, kept on the preparation itself)
+                if plain is None:
+                    plain = QKPreparation(rotation=Rotation(rot.inv_freq, rot.pairing, rot.rotary_dim, 1.0),
+                                          norm_eps=float(prep.norm_eps) / (m * m))
+                    prep._told_plainly = plain
+            return self.attention_from_qkv(rows, num_heads, num_kv_heads, head_dim, ctx.positions, ctx.token_segment,
+                                           plain, kv_cache, writes, slot_mapping, block_table, retention, scale, meta)
+        q = self.conv_qk_prepare(proj, bias, conv_w, taps, state, num_heads, num_kv_heads, head_dim, value_dim,
+                                 page_dim, prep, ctx, kv_cache if writes else None, slot_mapping)
+        return self.paged_attention(q, kv_cache, block_table, ctx.positions, ctx.token_segment, retention, scale, meta)
+
+    def conv_rows(self, proj, bias, conv_w, taps: int, state, ctx):
+        """``y[t] = sum_j conv_w[j] * u[t - taps + 1 + j]`` (``conv_w``: ``[taps, channels]``) with ``u = proj + bias`` rounded to the run dtype, rows
+        before a segment's start from the requests' two-halved state, whose other half gets the segment's last
+        ``taps - 1`` rows of ``u``; ``[N, C]`` in the run dtype.  See ``attention_conv.hip``."""
+        n, channels = proj.shape
+        dt = ctx.dtype
+        self._chk(proj, None, (n, channels), "projected rows")
+        if proj.dtype not in (dt, torch.float32):
+            raise KernelError(f"projected rows in {proj.dtype}, run dtype {dt}")
+        if bias is not None:
+            self._chk(bias, torch.float32, (channels,), "bias")
+        if taps:
+            self._chk(conv_w, torch.float32, (taps, channels), "convolution taps")
+        if taps > 1:
+            self._chk(state, dt, (state.shape[0], 2, taps - 1, channels), "convolution state")
+        for t, what, shape in ((ctx.token_segment, "token segments", (n,)),
+                               (ctx.cu_seqlens, "segment bounds", (ctx.num_segments + 1,)),
+                               (ctx.state_slots, "state slots", (ctx.num_segments,)),
+                               (ctx.state_phase, "state phases", (ctx.num_segments,))):
+            self._chk(t, torch.int32, shape, what)
+        y = torch.empty(n, channels, dtype=dt, device=proj.device)
+        self._call("jle_conv_rows", _p(proj), 1 if proj.dtype == torch.float32 else 0, _p(bias),
+                   _p(conv_w) if taps else None, int(taps), _p(state) if taps > 1 else None, _p(ctx.token_segment),
+                   _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(y),
+                   1 if dt == torch.bfloat16 else 0, n, ctx.num_segments, channels)
+        return y
 
     def conv_qk_prepare(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
                         value_dim: int, page_dim: int, prep, ctx, kv_cache, slot_mapping):
@@ -640,7 +698,7 @@ class HipOps:
         if bias is not None:
             self._chk(bias, torch.float32, (channels,), "bias")
         if taps:
-            self._chk(conv_w, torch.float32, (channels, taps), "convolution taps")
+            self._chk(conv_w, torch.float32, (taps, channels), "convolution taps")
         if taps > 1:
             self._chk(state, dt, (state.shape[0], 2, taps - 1, channels), "convolution state")
         rot = prep.rotation
@@ -863,6 +921,12 @@ class HipOps:
             return self.gemm_grouped(h, w, out_f32=True, tiled=tiled)
         return self.gemm(h, w, out_f32=True)
 
+    def softcap_(self, logits, cap: float):
+        """``cap * tanh(logits / cap)`` in place (float32)."""
+        self._chk(logits, torch.float32, None, "logits")
+        self._call("jle_softcap", _p(logits), logits.numel(), float(cap))
+        return logits
+
     def silu_mul(self, gate_up, activation: str = "silu"):
         n, f2 = gate_up.shape
         self._chk(gate_up, None, None, "gate|up")
@@ -924,8 +988,9 @@ class HipOps:
         hq, hk, dh = num_heads, num_kv_heads, head_dim
         ps = kv_cache.shape[3]
         group = hq // max(hk, 1)
+        whole_head = prep.rotation is None or (int(prep.rotation.rotary_dim) or dh) == dh
         if (meta is not None and meta.decode_bucket is not None and qkv.dtype == torch.bfloat16 and prep.plain
-                and group <= 32 and n * hk < self.TICKETS and 4 * (dh + 4 * group * (dh + 2)) <= 48 * 1024
+                and whole_head and group <= 32 and n * hk < self.TICKETS and 4 * (dh + 4 * group * (dh + 2)) <= 48 * 1024
                 and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
             self._chk(qkv, kv_cache.dtype, (n, (hq + 2 * hk) * dh), "q|k|v")
             self._chk(kv_cache, None, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")

@@ -154,15 +154,29 @@ class ReferenceOps:
             a = torch.nn.functional.silu(g)
         return (a * u).to(gate_up.dtype)
 
+    def softcap_(self, logits, cap: float):
+        """``cap * tanh(logits / cap)`` in place."""
+        return logits.copy_(torch.tanh(logits / cap) * cap)
+
     def sigmoid_mul(self, o, gate):
         """``o * sigmoid(gate)`` element by element (``gate``: a view with the same shape), float32 inside."""
         return (o.float() * torch.sigmoid(gate.float())).to(o.dtype)
+
+    def conv_attention(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
+                       value_dim: int, page_dim: int, prep, ctx, kv_cache, writes: bool, slot_mapping, block_table,
+                       retention, scale: float, meta=None):
+        """From the projected q|k|v rows to the attention output ``[N, num_heads * page_dim]``: bias, convolution
+        over time (with the requests' state), rotation and norm of q and k, pages written (if this run writes its
+        cache), attention over the pages; see :meth:`conv_qk_prepare`."""
+        q = self.conv_qk_prepare(proj, bias, conv_w, taps, state, num_heads, num_kv_heads, head_dim, value_dim,
+                                 page_dim, prep, ctx, kv_cache if writes else None, slot_mapping)
+        return self.paged_attention(q, kv_cache, block_table, ctx.positions, ctx.token_segment, retention, scale, meta)
 
     def conv_qk_prepare(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
                         value_dim: int, page_dim: int, prep, ctx, kv_cache, slot_mapping):
         """From the projected rows ``[N, Hq*dk + Hk*dk + Hk*dv]`` to prepared queries and written pages.
         ``u = proj + bias`` (rounded to the run dtype); every channel's causal convolution over time, ``y[t] =
-        sum_j conv_w[:, j] * u[t - taps + 1 + j]``, the rows before a segment's start from the request's state
+        sum_j conv_w[j] * u[t - taps + 1 + j]`` (``conv_w``: float32 ``[taps, channels]``), the rows before a segment's start from the request's state
         (``state[slot, phase]``: ``[taps - 1, channels]``, the oldest first; zeros before the sequence's start) -
         the last ``taps - 1`` rows of ``u`` go into ``state[slot, 1 - phase]``; ``y`` rounded to the run dtype; then
         q and k turned by ``prep.rotation`` (sines and cosines times its magnitude) and divided by their root mean
@@ -185,7 +199,7 @@ class ReferenceOps:
                 if taps > 1:
                     rows = torch.cat([state[slots[s], phase[s]].float(), rows], dim=0)  # [taps - 1 + len, C]
                 for j in range(taps):
-                    y[lo:hi] += w[:, j] * rows[j: j + hi - lo]
+                    y[lo:hi] += w[j] * rows[j: j + hi - lo]
                 if taps > 1:
                     state[slots[s], 1 - phase[s]] = rows[rows.shape[0] - (taps - 1):].to(state.dtype)
             y = y.to(dt).float()

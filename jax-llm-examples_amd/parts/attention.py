@@ -105,6 +105,8 @@ class Attention(Mixer):
         self.bias_run = None
         if self.biased:  # (the library's product adds a bias of its operands' dtype)
             self.bias_run = self.params["bqkv"].to(self.params["wqkv"].dtype)
+        # a tap's weights of all channels side by side, as the kernels read them
+        self.conv_by_tap = self.params["conv"].t().contiguous() if self.conv_taps else None
         self.wo_padded = None
         if self.page_dim != self.value_dim:  # the attention's output has page_dim elements a head: zeros' columns
             wo = self.params["wo"]
@@ -120,14 +122,13 @@ class Attention(Mixer):
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
         ops = ctx.ops
         if self.convolved:
-            # the projection (its bias added by the product where the library does it, else by the kernel below);
-            # then one kernel: convolution from the rows and the request's state, rotation, norm, pages
+            # the projection (its bias added by the product where the library does it, else by the kernel that reads
+            # the rows next); then convolution from the rows and the request's state, rotation, norm, pages, attention
             proj, bias = ops.linear_bias(h, self.params["wqkv"], self.params.get("bqkv"), self.bias_run)
-            q = ops.conv_qk_prepare(proj, bias, self.params.get("conv"), self.conv_taps, cache.state,
-                                    self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, self.page_dim,
-                                    self.prep, ctx, cache.kv if cache.writes else None, cache.slot_mapping)
-            o = ops.paged_attention(q, cache.kv, cache.block_table, ctx.positions, ctx.token_segment, self.retention,
-                                    self.softmax_scale, cache.attn_meta)
+            o = ops.conv_attention(proj, bias, self.conv_by_tap, self.conv_taps, cache.state, self.num_heads,
+                                   self.num_kv_heads, self.head_dim, self.value_dim, self.page_dim, self.prep, ctx,
+                                   cache.kv, cache.writes, cache.slot_mapping, cache.block_table, self.retention,
+                                   self.softmax_scale, cache.attn_meta)
             return ops.linear(o, self.params["wo"] if self.wo_padded is None else self.wo_padded)
         qkv = ops.linear(h, self.params["wqkv"])
         o = ops.attention_from_qkv(

@@ -104,5 +104,5 @@ class LinearHead(OutputHead):
         if self.biased:
             logits.add_(self.params["bias"])
         if self.softcap is not None:
-            logits = torch.tanh(logits / self.softcap) * self.softcap
+            logits = ctx.ops.softcap_(logits, self.softcap)
         return logits

@@ -22,7 +22,7 @@ from ..weights.bindings import TensorBinding
 class TiradraArchitecture:
     names = ("Tiradra", "tiradra")
     # what of csrc/ a model of this design calls (a first run on a machine without a built library compiles these)
-    kernel_sources = ("elementwise.hip", "parallel.hip", "attention_conv.hip", "attention_latent.hip",
+    kernel_sources = ("elementwise.hip", "parallel.hip", "attention_conv.hip", "attention_prep.hip", "attention_latent.hip",
                       "attention_mfma.hip", "attention_generic.hip", "attention_f32.hip", "gemm_skinny.hip",
                       "gemm_stream.hip", "gemm_grouped.hip", "gemm_generic.hip", "sampling.hip")
 

@@ -172,7 +172,7 @@ def test_convolution_rotation_norm_and_pages_alone(device, taps, dk, dv, rd):
         rows = dev(torch.cat([proj[k][a:b] for k, a, b in cut]))
         slots = torch.tensor([pages_of[k][t // ps] * ps + t % ps for k, a, b in cut for t in range(a, b)],
                              dtype=torch.int32, device=device)
-        args = (rows, dev(bias), dev(w) if taps else None, taps, state, hq, hk, dk, dv, D, prep, ctx, kv, slots)
+        args = (rows, dev(bias), dev(w.t().contiguous()) if taps else None, taps, state, hq, hk, dk, dv, D, prep, ctx, kv, slots)
         q1 = ops.conv_qk_prepare(*args).clone()
         q2 = ops.conv_qk_prepare(*args)  # (again before the commit: the half it reads was not written)
         assert torch.equal(q1, q2)
@@ -191,6 +191,41 @@ def test_convolution_rotation_norm_and_pages_alone(device, taps, dk, dv, rd):
             val = kv[page, 1].view(hk, D, ps)[:, :, off].cpu()
             assert torch.allclose(key[:, :dk], want[k][1][t], rtol=2e-4, atol=2e-5) and (key[:, dk:] == 0).all()
             assert torch.allclose(val[:, :dv], want[k][2][t], rtol=2e-4, atol=2e-5) and (val[:, dv:] == 0).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("taps,channels", [(4, 256), (3, 100), (2, 64), (5, 8), (1, 24), (0, 40)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_convolution_kernel_alone(taps, channels, dtype):
+    """The kernel that convolves and does nothing else (rows that the plain preparation kernels take afterwards),
+    eight channels a thread or one: portions shorter than the taps, the state's halves, a step run twice."""
+    ops = _ops("cuda:0")
+    g = torch.Generator().manual_seed(taps + channels)
+    lens = {"a": 23, "b": 9}
+    proj = {k: torch.randn(n, channels, generator=g).to(dtype) for k, n in lens.items()}
+    bias, w = torch.randn(channels, generator=g) * 0.3, (torch.randn(max(taps, 1), channels, generator=g) * 0.6)
+    want = {}
+    for k in lens:
+        u = (proj[k].float() + bias).to(dtype).double()
+        want[k] = (P.causal_conv(u, w.t().double()) if taps else u).float()
+    dev = lambda t: t.to("cuda:0")
+    state = torch.zeros(3, 2, max(taps - 1, 1), channels, device="cuda:0", dtype=dtype) if taps > 1 else None
+    cuts = [[("a", 0, 5)], [("a", 5, 7), ("b", 0, 2)], [("b", 2, 9), ("a", 7, 8)], [("a", 8, 9)], [("a", 9, 23)]]
+    slot, steps_done, got = {"a": 2, "b": 0}, {"a": 0, "b": 0}, {k: [] for k in lens}
+    for cut in cuts:
+        ctx = _step_ctx("cuda:0", [b - a for _, a, b in cut], [a for _, a, _ in cut], [slot[k] for k, _, _ in cut],
+                        [steps_done[k] & 1 for k, _, _ in cut], dtype=dtype)
+        rows = dev(torch.cat([proj[k][a:b] for k, a, b in cut]))
+        y1 = ops.conv_rows(rows, dev(bias), dev(w) if taps else None, taps, state, ctx).clone()
+        assert torch.equal(y1, ops.conv_rows(rows, dev(bias), dev(w) if taps else None, taps, state, ctx))
+        o = 0
+        for k, a, b in cut:
+            got[k].append(y1[o:o + b - a].float().cpu())
+            o += b - a
+            steps_done[k] += 1
+    tol = dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    for k in lens:
+        assert torch.allclose(torch.cat(got[k]), want[k], **tol), (torch.cat(got[k]) - want[k]).abs().max()
 
 
 def _mixer_alone(folder, device, layer, sizes, x, dtype="float32", page_size=16, sink=None):
