@@ -64,7 +64,8 @@ def load_model(model_dir, dtype="bfloat16", device="cuda:0") -> DecoderModel:
     model.allocate()
     load_weights(model, os.fspath(model_dir), arch.bindings(cfg, model.plan),
                  optional_prefixes=getattr(arch, "optional_prefixes", ()),
-                 ignored_prefixes=getattr(arch, "ignored_prefixes", ()))  # (finalizes the model's parts)
+                 ignored_prefixes=tuple(getattr(arch, "ignored_prefixes", ())) +
+                 tuple(arch.unused_prefixes(cfg) if hasattr(arch, "unused_prefixes") else ()))
     return model
 
 

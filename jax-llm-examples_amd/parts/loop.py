@@ -30,7 +30,11 @@ def build_loop(spec):
 @register_loop("pass_entry")
 class PassEntry(Part):
     graph_safe = True
-    needs_embedding_output = True  # the model keeps a copy of the embedding's output for it
+
+    @property
+    def needs_embedding_output(self) -> bool:
+        """Whether the model has to keep a copy of the embedding's output for it (a single pass adds none)."""
+        return self.times > 1
 
     def __init__(self, spec) -> None:
         super().__init__()

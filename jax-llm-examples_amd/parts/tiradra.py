@@ -35,6 +35,11 @@ class TiradraArchitecture:
     def config_to_dict(self, cfg: TiradraConfig, architecture: str | None = None) -> dict:
         return cfg.to_dict(architecture or "Tiradra")
 
+    def unused_prefixes(self, cfg: TiradraConfig) -> tuple:
+        """Tensors that a checkpoint may hold and this model does not read: the feed-forward's norm of a layer that
+        has no feed-forward."""
+        return tuple(f"l{i}.norm2" for i, lc in enumerate(cfg.layers) if lc.mlp is None)
+
     def bindings(self, cfg: TiradraConfig, plan: ModelPlan) -> list[TensorBinding]:
         D, V = cfg.width, cfg.vocab
         mat = lambda fan_in: ("normal", 1.0 / math.sqrt(fan_in))

@@ -633,3 +633,18 @@ def test_weights_error_names_what_is_missing(folders, tmp_path):
     with pytest.raises(WeightsError) as e:
         load_model(str(tmp_path / "m"), "float32", "cpu")
     assert e.value.missing == ["l0.mix.k.conv"] and e.value.unexpected == ["l2.mix.v.conv"]
+
+
+def test_a_norm_nobody_reads_is_let_be(folders, tmp_path):
+    """A checkpoint may hold the second norm of a layer that has no feed-forward."""
+    from safetensors.torch import load_file, save_file
+
+    w = load_file(os.path.join(folders["TA"], "model.safetensors"))
+    assert "l2.norm2" not in w
+    w["l2.norm2"] = torch.zeros(64)
+    (tmp_path / "m").mkdir()
+    save_file(w, str(tmp_path / "m" / "model.safetensors"))
+    with open(os.path.join(folders["TA"], "config.json")) as f:
+        (tmp_path / "m" / "config.json").write_text(f.read())
+    model = load_model(str(tmp_path / "m"), "float32", "cpu")
+    assert "layers.2.feed_forward_norm.weight" not in model.named_parameters()
