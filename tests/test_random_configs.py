@@ -2,7 +2,8 @@
 widths and vocabularies that are no power of two, one to seventeen experts with one or two per token, dense layers
 between them, chunks that are no multiple of the page size, three page sizes, with and without frequency scaling,
 q/k norm and temperature.  Each runs a mixed trace (portions beside single tokens, pages used again) in float32 and
-bfloat16 against the plain implementation: the kernels take every size the configuration allows."""
+bfloat16 against the plain implementation: the kernels take every size the configuration allows.  The same for the
+Tiradra design (``draw_tiradra``)."""
 import random
 
 import pytest
@@ -64,4 +65,85 @@ def test_random_configuration(tmp_path, seed, dtype):
         assert torch.isfinite(got[rid]).all(), f"{top}: {rid}: non-finite logits"
         err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
         bad = (err > TOL[dtype]).nonzero().squeeze(-1).tolist()
+        assert not bad, f"{top}, page size {page_size}: {rid}: first wrong position {bad[0]}, error {err[bad[0]]:.3g}"
+
+
+# ---------------------------------------------------------------------------------------------- the Tiradra design
+def draw_tiradra(seed: int):
+    """Every size and option of the design at random: head sizes that are and are not multiples of 8 or 16, values
+    smaller and larger than keys, one to eight query heads a kv head, none to six taps, rotations over part of a
+    head with and without a stretch, latents that do and do not fit the matrix-core kernels, loops anywhere, with
+    and without the pair table and the cap, layers without a feed-forward."""
+    rng = random.Random(1000 + seed)
+    width = rng.choice([40, 54, 64, 72, 96, 128, 136, 200, 256])
+
+    def rot(limit):
+        dims = rng.choice([d for d in (2, 4, 6, 8, 16, 24, 32, 48, 64, 96, 128) if d <= limit] + [limit - limit % 2])
+        r = {"base": rng.choice([50.0, 10000.0, 500000.0]), "dims": max(dims, 2)}
+        if rng.random() < 0.6:
+            r["scaling"] = {"factor": rng.choice([1.5, 2.0, 4.0, 32.0]), "original": rng.choice([16, 64, 2048]),
+                            "fast": rng.choice([4.0, 32.0]), "slow": rng.choice([0.5, 1.0, 2.0])}
+        return r
+
+    def attention():
+        kv = rng.choice([1, 2, 3, 4])
+        dim = rng.choice([6, 8, 16, 20, 32, 48, 64, 80, 96, 128])
+        m = {"heads": kv * rng.choice([1, 2, 3, 8]), "kv_heads": kv, "dim": dim,
+             "vdim": rng.choice([dim, dim, 4, 8, 24, 64, 128]), "scale": rng.choice([dim ** -0.5, 0.3, 0.7]),
+             "rot": rot(dim)}
+        taps = rng.choice([0, 1, 2, 3, 4, 4, 6])
+        if taps:
+            m["conv"] = taps
+        return "attention", m
+
+    def latent():
+        rot_dim = rng.choice([2, 4, 8, 16, 24, 32, 64, 72])
+        r = rot(rot_dim)
+        r["dims"] = rot_dim  # (the rotated part turns as a whole)
+        return "latent_attention", {"heads": rng.choice([1, 2, 3, 6, 16, 20]), "dim": rng.choice([4, 8, 16, 40, 64]),
+                                    "rot_dim": rot_dim, "vdim": rng.choice([4, 8, 24, 64]),
+                                    "kv_rank": rng.choice([12, 16, 18, 32, 64, 96, 128, 160, 192]),
+                                    "scale": rng.choice([0.1, 0.25, 0.5]), "rot": r}
+
+    layers = []
+    for _ in range(rng.randint(1, 5)):
+        kind, mixer = rng.choice([attention, attention, latent])()
+        ff = rng.choice([None, 24, 32, 40, 64, 128, 320])
+        layers.append({"type": kind, "mixer": mixer, "mlp": None if ff is None else {"kind": "dense", "ff": ff}})
+    top = {"architecture": "Tiradra", "vocab": rng.choice([97, 257, 300, 512, 1001]), "width": width,
+           "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])}, "layers": layers}
+    if rng.random() < 0.75:
+        top["embedding"] = {"bigram": {"buckets": rng.choice([1, 13, 1000, 65521]), "mul_prev": rng.choice([0, 1, 31, 10 ** 9 + 7]),
+                                       "mul_cur": rng.choice([1, 17, 10 ** 9 + 9])}}
+    if rng.random() < 0.75:
+        start = rng.randint(0, len(layers) - 1)
+        top["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.choice([1, 2, 2, 3])}
+    if rng.random() < 0.7:
+        top["logit_softcap"] = rng.choice([5.0, 15.0, 50.0])
+    lengths = [rng.choice([1, 2, 17, 33, 64, 65, 97, 130]) for _ in range(rng.randint(2, 5))]
+    return top, rng.choice([16, 16, 32, 64]), lengths
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_random_tiradra_configuration(tmp_path, seed, dtype):
+    from plain_tiradra import PlainTiradra
+
+    top, page_size, lengths = draw_tiradra(seed)
+    arch = get_architecture(top["architecture"])
+    folder = write_random_model(arch, arch.parse_config(top), str(tmp_path / "m"), seed,
+                                torch.float32 if dtype == "float32" else torch.bfloat16)
+    reqs = traces.random_requests(top["vocab"], lengths, seed=seed)
+    steps = traces.mixed(reqs, seed=seed)
+    runner = make_runner(folder, dtype, traces.max_live_tokens(steps), "cuda:0", page_size=page_size, poison=True,
+                         max_requests=4)
+    got = traces.run_trace(runner, steps)
+    runner.cache.check()
+    assert runner.cache.num_live() == 0
+    plain = PlainTiradra(folder)
+    for rid, toks in reqs.items():
+        ref = plain.logits(toks).float()
+        assert torch.isfinite(got[rid]).all(), f"{top}: {rid}: non-finite logits"
+        err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
+        bad = (err > {"float32": 3e-5, "bfloat16": 5e-2}[dtype]).nonzero().squeeze(-1).tolist()
         assert not bad, f"{top}, page size {page_size}: {rid}: first wrong position {bad[0]}, error {err[bad[0]]:.3g}"
