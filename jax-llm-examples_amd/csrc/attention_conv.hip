@@ -230,8 +230,16 @@ __device__ __forceinline__ void projected8(const ConvArgs<PT, T>& a, size_t row,
   for (int i = 0; i < 8; ++i) u[i] = Num<T>::round(u[i] + bias8[i]);
 }
 
+constexpr int kRowsPerBlock = 8;  // tokens a block of the eight-channel kernel takes in a step of many tokens
+constexpr int kTapsInRegisters = 8;
+
+// A block takes rows_per_block consecutive tokens of the step for its channels (one in a step of few tokens, where
+// the blocks are few as it is): the taps' weights and the bias are read once per block (up to kTapsInRegisters taps;
+// more are read again for every token), and the rows that neighbouring tokens share come from the first-level
+// cache.  A token's sums are the same whatever the number.
 template <typename PT, typename T>
-__global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T* __restrict__ y_out, int N) {
+__global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T* __restrict__ y_out, int N,
+                                                            int token_blocks, int rows_per_block) {
   const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c >= a.C) return;
   const int K = a.taps;
@@ -240,9 +248,9 @@ __global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T
   for (int i = 0; i < 8; ++i) bias8[i] = 0.f;
   if (a.bias != nullptr) Row8<float>::load(a.bias + c, bias8);
   float u[8];
-  if ((int)blockIdx.x >= N) {  // a segment's state
+  if ((int)blockIdx.x >= token_blocks) {  // a segment's state
     if (K <= 1) return;
-    const int seg = blockIdx.x - N;
+    const int seg = blockIdx.x - token_blocks;
     const int row0 = a.cu_seqlens[seg], len = a.cu_seqlens[seg + 1] - row0;
     const size_t slot = (size_t)a.state_slots[seg];
     const int phase = a.state_phase[seg];
@@ -256,38 +264,58 @@ __global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T
     }
     return;
   }
-  const int n = blockIdx.x;
-  float y[8];
-  if (K == 0) {
-    projected8(a, (size_t)n, c, bias8, y);
-  } else {
-    const int seg = a.token_segment[n];
-    const int t = n - a.cu_seqlens[seg];
-    const T* old = nullptr;
-    if (K > 1) old = a.state + ((size_t)a.state_slots[seg] * 2 + a.state_phase[seg]) * (K - 1) * a.C;
+  float wreg[kTapsInRegisters][8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) y[i] = 0.f;
-    for (int j = 0; j < K; ++j) {
-      const int back = K - 1 - j;
-      if (t - back >= 0) projected8(a, (size_t)(n - back), c, bias8, u);
-      else Row8<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c, u);
-      float w8[8];
-      Row8<float>::load(a.w + (size_t)j * a.C + c, w8);
+  for (int j = 0; j < kTapsInRegisters; ++j)
+    if (j < K) Row8<float>::load(a.w + (size_t)j * a.C + c, wreg[j]);
+  const int n_end = min(N, ((int)blockIdx.x + 1) * rows_per_block);
+  for (int n = blockIdx.x * rows_per_block; n < n_end; ++n) {
+    float y[8];
+    if (K == 0) {
+      projected8(a, (size_t)n, c, bias8, y);
+    } else {
+      const int seg = a.token_segment[n];
+      const int t = n - a.cu_seqlens[seg];
+      const T* old = nullptr;
+      if (K > 1) old = a.state + ((size_t)a.state_slots[seg] * 2 + a.state_phase[seg]) * (K - 1) * a.C;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = __builtin_fmaf(w8[i], u[i], y[i]);
+      for (int i = 0; i < 8; ++i) y[i] = 0.f;
+#pragma unroll
+      for (int j = 0; j < kTapsInRegisters; ++j) {  // (the taps ascending, as in every kernel of this file)
+        if (j < K) {
+          const int back = K - 1 - j;
+          if (t - back >= 0) projected8(a, (size_t)(n - back), c, bias8, u);
+          else Row8<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c, u);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) y[i] = __builtin_fmaf(wreg[j][i], u[i], y[i]);
+        }
+      }
+      for (int j = kTapsInRegisters; j < K; ++j) {
+        const int back = K - 1 - j;
+        if (t - back >= 0) projected8(a, (size_t)(n - back), c, bias8, u);
+        else Row8<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c, u);
+        float w8[8];
+        Row8<float>::load(a.w + (size_t)j * a.C + c, w8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = __builtin_fmaf(w8[i], u[i], y[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = Num<T>::round(y[i]);
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) y[i] = Num<T>::round(y[i]);
+    Row8<T>::store(y_out + (size_t)n * a.C + c, y);
   }
-  Row8<T>::store(y_out + (size_t)n * a.C + c, y);
 }
 
 template <typename PT, typename T>
 int launch_conv_rows(const ConvArgs<PT, T>& a, void* y_out, int N, int R, hipStream_t s) {
   const uintptr_t all = (uintptr_t)a.proj | (uintptr_t)a.bias | (uintptr_t)a.w | (uintptr_t)a.state | (uintptr_t)y_out;
   if (a.C % 8 == 0 && all % 16 == 0)  // (by the sizes alone: the same kernel for every step of a model)
-    hipLaunchKernelGGL((conv_rows_vec_kernel<PT, T>), dim3(N + (a.taps > 1 ? R : 0), (a.C / 8 + 255) / 256), dim3(256),
-                       0, s, a, (T*)y_out, N);
+  {
+    const int per = N >= 512 ? kRowsPerBlock : 1;
+    const int token_blocks = (N + per - 1) / per;
+    hipLaunchKernelGGL((conv_rows_vec_kernel<PT, T>), dim3(token_blocks + (a.taps > 1 ? R : 0), (a.C / 8 + 255) / 256),
+                       dim3(256), 0, s, a, (T*)y_out, N, token_blocks, per);
+  }
   else
     hipLaunchKernelGGL((conv_rows_kernel<PT, T>), dim3(N + (a.taps > 1 ? R : 0), (a.C + 255) / 256), dim3(256), 0, s, a,
                        (T*)y_out, N);

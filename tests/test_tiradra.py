@@ -226,6 +226,16 @@ def test_convolution_kernel_alone(taps, channels, dtype):
     tol = dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
     for k in lens:
         assert torch.allclose(torch.cat(got[k]), want[k], **tol), (torch.cat(got[k]) - want[k]).abs().max()
+    # a step of many tokens (several tokens a block) gives every token the bits it gets in a step of its own
+    n = 700
+    rows = dev(torch.randn(n, channels, generator=g).to(dtype))
+    fresh = lambda: torch.zeros(1, 2, max(taps - 1, 1), channels, device="cuda:0", dtype=dtype) if taps > 1 else None
+    whole = ops.conv_rows(rows, dev(bias), dev(w) if taps else None, taps, fresh(), _step_ctx("cuda:0", [n], [0], [0], [0], dtype))
+    st, parts = fresh(), []
+    for i, (lo, hi) in enumerate([(0, 300), (300, 301), (301, 700)]):
+        ctx = _step_ctx("cuda:0", [hi - lo], [lo], [0], [i & 1], dtype)
+        parts.append(ops.conv_rows(rows[lo:hi].contiguous(), dev(bias), dev(w) if taps else None, taps, st, ctx))
+    assert torch.equal(whole, torch.cat(parts))
 
 
 def _mixer_alone(folder, device, layer, sizes, x, dtype="float32", page_size=16, sink=None):
