@@ -61,7 +61,7 @@ def design_configs(size: dict, layers: int):
     t_attn = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
               "rot": {"base": 500000.0, "dims": 128, "scaling": yarn}}
     tiradra = {"architecture": "Tiradra", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
-               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "logit_softcap": 30.0,
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 37, "mul_cur": 11}}, "logit_softcap": 30.0,
                "layers": [{"type": "attention" if i % 4 else "latent_attention", "mixer": t_attn if i % 4 else t_latent,
                            "mlp": {"kind": "dense", "ff": size["ff"]}} for i in range(layers)]}
     if layers >= 3:
